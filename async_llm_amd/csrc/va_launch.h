@@ -1,0 +1,48 @@
+// Kernel argument blocks and launchers shared between translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "va_device.h"
+
+namespace va {
+
+struct AttnArgs {
+  const void* q;
+  long long q_row_stride;  // elements between query rows
+  const void* k_pool;
+  const void* v_pool;
+  long long pool_row_stride;  // elements between token slots
+  const int32_t* items;
+  const int32_t* links;
+  const int32_t* qrefs;
+  const int32_t* kv_indices;
+  const int64_t* sub_worker;
+  const int64_t* sub_loc;
+  long long sub_loc_axis_stride;
+  void* out;
+  float* lse;
+  int lse_base2;
+  float* part_acc;  // [n_partials, Hq, D]
+  float* part_ml;   // [n_partials, Hq, 2]  (running max in log2 units, sum)
+  int num_q_heads, num_kv_heads, head_dim, page_size;
+  RopeDev rope;
+  float scale_log2;  // log2(e) / sqrt(head_dim)
+};
+
+struct MergeArgs {
+  const int32_t* row_indptr;
+  const int32_t* row_ids;
+  const int32_t* row_flags;
+  const float* part_acc;
+  const float* part_ml;
+  void* out;
+  float* lse;
+  int lse_base2;
+  int num_q_heads, head_dim;
+};
+
+// Matrix-core attention (va_mfma.hip).
+int launch_mfma(const AttnArgs& a, int dtype, int n_items, int q_tile, hipStream_t stream);
+
+}  // namespace va

@@ -1,0 +1,429 @@
+// Host-side work decomposition for view attention.
+//
+// Takes the planned sub-request tables of one launch (what the reference feeds
+// to FlashInfer's plan(): python/minisgl/shared_cache/attention.py:390-426 for
+// decode, :574-604 for prefill) and cuts them into work items sized for the
+// 256 CUs of an MI355X:
+//   * stand-alone (decode) sub-requests that read the identical page list are
+//     batched into one query tile, so a block shared by many views is streamed
+//     once per tile instead of once per reader;
+//   * long KV runs are split into chunks (split-KV); every (row, chunk) yields a
+//     partial softmax state that the merge kernel folds together with the
+//     row's other segments -- the same LSE merge the reference performs across
+//     segments (attention.py:694-703);
+//   * the sub-requests of one prefill request are chained so a query tile walks
+//     all of its segments in one workgroup, carrying the online softmax in
+//     registers (no per-segment scratch as in attention.py:736-751).
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <numeric>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/viewattn.h"
+#include "va_internal.h"
+#include "va_plan.h"
+
+namespace {
+
+struct Item {
+  int32_t link_begin, n_links, n_q, part_base, tokens;
+};
+struct Link {
+  int32_t kv_begin, tok_begin, tok_end, qref, causal_base, flags;
+};
+
+struct Built {
+  std::vector<Item> items;
+  std::vector<Link> links;
+  std::vector<int32_t> qrefs;
+  std::vector<int32_t> row_indptr;
+  std::vector<int32_t> row_ids;
+  std::vector<int32_t> row_flags;
+  int32_t n_partials = 0;
+  int32_t kernel = 0, q_tile = 0, kv_chunk = 0;
+};
+
+inline int32_t round_up(int64_t x, int32_t m) { return (int32_t)(((x + m - 1) / m) * m); }
+
+int check_subs(const VaSubRequests* s, const VaShape* shape) {
+  if (!s || !shape) return va_fail(VA_ERR_ARG, "null argument");
+  if (s->n_sub < 0 || s->n_rows < 0 || s->n_subrows < 0) return va_fail(VA_ERR_ARG, "negative count");
+  if (s->n_sub > 0 && (!s->qo_indptr || !s->kv_indptr || !s->seq_lens || !s->flags || !s->chain))
+    return va_fail(VA_ERR_ARG, "null sub-request table");
+  if (s->n_subrows > 0 && !s->sub_worker) return va_fail(VA_ERR_ARG, "null sub_worker");
+  if (shape->num_kv_heads <= 0 || shape->num_q_heads % shape->num_kv_heads)
+    return va_fail(VA_ERR_ARG, "num_q_heads must be a multiple of num_kv_heads");
+  if (shape->page_size <= 0) return va_fail(VA_ERR_ARG, "page_size must be positive");
+  if (s->n_sub > 0) {
+    if (s->qo_indptr[0] != 0 || s->kv_indptr[0] != 0) return va_fail(VA_ERR_ARG, "indptr must start at 0");
+    if (s->qo_indptr[s->n_sub] != s->n_subrows)
+      return va_fail(VA_ERR_ARG, "qo_indptr[-1]=%d != n_subrows=%d", s->qo_indptr[s->n_sub], s->n_subrows);
+  }
+  for (int32_t i = 0; i < s->n_sub; ++i) {
+    const int32_t nq = s->qo_indptr[i + 1] - s->qo_indptr[i];
+    const int32_t ne = s->kv_indptr[i + 1] - s->kv_indptr[i];
+    if (nq < 0 || ne < 0) return va_fail(VA_ERR_ARG, "indptr not monotone at sub-request %d", i);
+    const int32_t len = s->seq_lens[i];
+    const int64_t cap = (s->flags[i] & VA_SUB_SLOTS) ? ne : (int64_t)ne * shape->page_size;
+    if (len < 0 || len > cap)
+      return va_fail(VA_ERR_ARG, "sub-request %d: seq_len %d does not fit its %d kv entries", i, len, ne);
+    if ((s->flags[i] & VA_SUB_CAUSAL) && nq > len)
+      return va_fail(VA_ERR_ARG, "sub-request %d: causal with more query rows (%d) than keys (%d)", i, nq, len);
+    if (ne > 0 && !s->kv_indices) return va_fail(VA_ERR_ARG, "null kv_indices");
+  }
+  for (int32_t i = 0; i < s->n_subrows; ++i)
+    if (s->sub_worker[i] < 0 || s->sub_worker[i] >= s->n_rows)
+      return va_fail(VA_ERR_ARG, "sub_worker[%d]=%lld outside [0,%d)", i, (long long)s->sub_worker[i], s->n_rows);
+  return VA_OK;
+}
+
+int resolve_kernel(const VaShape* shape, const VaPlanParams* p) {
+  int kernel = p ? p->kernel : VA_KERNEL_AUTO;
+  const int g = shape->num_q_heads / shape->num_kv_heads;
+  const bool mfma_ok = va_mfma_supported(shape->dtype, shape->head_dim, g);
+  if (kernel == VA_KERNEL_AUTO) kernel = mfma_ok ? VA_KERNEL_MFMA : VA_KERNEL_GENERIC;
+  if (kernel == VA_KERNEL_MFMA && !mfma_ok) return -1;
+  if (kernel != VA_KERNEL_MFMA && kernel != VA_KERNEL_GENERIC) return -1;
+  return kernel;
+}
+
+// Visible tokens of a causal/non-causal sub-request for tile rows [a, b).
+inline int32_t visible_end(int32_t len, int32_t nq, bool causal, int32_t b) {
+  return causal ? std::min(len, len - nq + b) : len;
+}
+
+int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* params, Built& out) {
+  int rc = check_subs(s, shape);
+  if (rc) return rc;
+  const int kernel = resolve_kernel(shape, params);
+  if (kernel < 0) return va_fail(VA_ERR_ARG, "requested kernel family does not support this dtype/shape");
+  const int g = shape->num_q_heads / shape->num_kv_heads;
+  int q_tile = params && params->q_tile > 0 ? params->q_tile : 0;
+  const int q_tile_max = kernel == VA_KERNEL_MFMA ? va_mfma_max_q_tile(g) : 64;
+  const bool has_chain = std::any_of(s->chain, s->chain + s->n_sub, [](int32_t c) { return c >= 0; });
+  if (q_tile == 0) q_tile = kernel == VA_KERNEL_MFMA ? va_mfma_default_q_tile(g, has_chain) : 1;
+  if (q_tile > q_tile_max) return va_fail(VA_ERR_ARG, "q_tile %d exceeds the kernel's maximum %d", q_tile, q_tile_max);
+  const int target = params && params->target_items > 0 ? params->target_items
+                                                        : std::max(64, 2048 / shape->num_kv_heads);
+  const int gran = 64;  // chunk boundaries are multiples of this many tokens
+
+  // ---- stand-alone sub-requests: batch readers of identical KV lists ----
+  struct Group {
+    int32_t rep;                  // representative sub-request
+    std::vector<int32_t> subrows; // sub-row ids of all members, in order
+  };
+  std::vector<Group> groups;
+  {
+    std::unordered_map<uint64_t, std::vector<int32_t>> by_hash;  // hash -> group ids
+    for (int32_t i = 0; i < s->n_sub; ++i) {
+      if (s->chain[i] >= 0) continue;
+      const int32_t nq = s->qo_indptr[i + 1] - s->qo_indptr[i];
+      if (nq == 0 || s->seq_lens[i] == 0) continue;
+      if (s->flags[i] & VA_SUB_CAUSAL)
+        return va_fail(VA_ERR_ARG, "sub-request %d: causal sub-requests must belong to a chain", i);
+      const int32_t b = s->kv_indptr[i], ne = s->kv_indptr[i + 1] - b;
+      int32_t gid = -1;
+      uint64_t h = 0;
+      if (q_tile > 1) {
+        h = (uint64_t)(uint32_t)s->kv_indices[b] * 0x9E3779B97F4A7C15ull ^
+            ((uint64_t)(uint32_t)s->seq_lens[i] << 32) ^ (uint64_t)(uint32_t)(ne * 31 + s->flags[i]);
+        auto it = by_hash.find(h);
+        if (it != by_hash.end()) {
+          for (int32_t cand : it->second) {
+            const int32_t r = groups[cand].rep;
+            const int32_t rb = s->kv_indptr[r], rn = s->kv_indptr[r + 1] - rb;
+            if (rn == ne && s->seq_lens[r] == s->seq_lens[i] && s->flags[r] == s->flags[i] &&
+                !std::memcmp(s->kv_indices + rb, s->kv_indices + b, sizeof(int32_t) * ne)) {
+              gid = cand;
+              break;
+            }
+          }
+        }
+      }
+      if (gid < 0) {
+        gid = (int32_t)groups.size();
+        groups.push_back(Group{i, {}});
+        if (q_tile > 1) by_hash[h].push_back(gid);
+      }
+      for (int32_t r = s->qo_indptr[i]; r < s->qo_indptr[i + 1]; ++r) groups[gid].subrows.push_back(r);
+    }
+  }
+
+  // ---- chains: sub-requests of one prefill request, in table order ----
+  std::vector<std::vector<int32_t>> chains;
+  {
+    std::unordered_map<int32_t, int32_t> chain_index;
+    for (int32_t i = 0; i < s->n_sub; ++i) {
+      const int32_t c = s->chain[i];
+      if (c < 0) continue;
+      auto it = chain_index.find(c);
+      if (it == chain_index.end()) {
+        it = chain_index.emplace(c, (int32_t)chains.size()).first;
+        chains.emplace_back();
+      }
+      chains[it->second].push_back(i);
+    }
+    for (auto& ch : chains) {
+      const int32_t nq = s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]];
+      for (int32_t m : ch) {
+        if (s->qo_indptr[m + 1] - s->qo_indptr[m] != nq)
+          return va_fail(VA_ERR_ARG, "chain %d: members disagree on the number of query rows", s->chain[m]);
+        for (int32_t r = 0; r < nq; ++r)
+          if (s->sub_worker[s->qo_indptr[m] + r] != s->sub_worker[s->qo_indptr[ch[0]] + r])
+            return va_fail(VA_ERR_ARG, "chain %d: members disagree on output rows", s->chain[m]);
+      }
+    }
+  }
+
+  // ---- total tokens -> chunk size for split-KV ----
+  int64_t total_tokens = 0;
+  int64_t n_group_tiles = 0;
+  for (auto& gr : groups) {
+    const int64_t tiles = ((int64_t)gr.subrows.size() + q_tile - 1) / q_tile;
+    n_group_tiles += tiles;
+    total_tokens += tiles * s->seq_lens[gr.rep];
+  }
+  int64_t chain_tiles = 0, chain_tokens = 0;
+  for (auto& ch : chains) {
+    const int32_t nq = s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]];
+    for (int32_t a = 0; a < nq; a += q_tile) {
+      const int32_t b = std::min(nq, a + q_tile);
+      ++chain_tiles;
+      for (int32_t m : ch)
+        chain_tokens += visible_end(s->seq_lens[m], nq, s->flags[m] & VA_SUB_CAUSAL, b);
+    }
+  }
+  total_tokens += chain_tokens;
+  int32_t kv_chunk = params && params->kv_chunk > 0 ? round_up(params->kv_chunk, gran) : 0;
+  if (kv_chunk == 0) {
+    const int64_t per_item = (total_tokens + target - 1) / target;
+    kv_chunk = round_up(std::max<int64_t>(per_item, 4 * gran), gran);
+  }
+
+  out.kernel = kernel;
+  out.q_tile = q_tile;
+  out.kv_chunk = kv_chunk;
+
+  // contributions per output row decide direct-vs-partial
+  std::vector<int32_t> row_count(s->n_rows, 0);
+  struct Pending {
+    int32_t item;
+    std::vector<int32_t> rows;  // output row per tile row
+  };
+  std::vector<Pending> pend;
+
+  auto emit = [&](int32_t n_q, const std::vector<Link>& links, std::vector<int32_t>&& rows) {
+    int32_t tokens = 0;
+    for (auto& l : links) tokens += l.tok_end - l.tok_begin;
+    Item it{(int32_t)out.links.size(), (int32_t)links.size(), n_q, -1, tokens};
+    out.links.insert(out.links.end(), links.begin(), links.end());
+    for (int32_t r : rows) ++row_count[r];
+    pend.push_back(Pending{(int32_t)out.items.size(), std::move(rows)});
+    out.items.push_back(it);
+  };
+
+  for (auto& gr : groups) {
+    const int32_t rep = gr.rep;
+    const int32_t len = s->seq_lens[rep];
+    const int32_t n_chunks = (len + kv_chunk - 1) / kv_chunk;
+    const int32_t per = round_up((len + n_chunks - 1) / n_chunks, gran);
+    const int32_t lflags = VA_LINK_INDIRECT | ((s->flags[rep] & VA_SUB_SLOTS) ? VA_LINK_SLOTS : 0);
+    for (size_t a = 0; a < gr.subrows.size(); a += q_tile) {
+      const size_t b = std::min(gr.subrows.size(), a + (size_t)q_tile);
+      const int32_t qref = (int32_t)out.qrefs.size();
+      out.qrefs.insert(out.qrefs.end(), gr.subrows.begin() + a, gr.subrows.begin() + b);
+      for (int32_t t0 = 0; t0 < len; t0 += per) {
+        std::vector<int32_t> rows;
+        for (size_t r = a; r < b; ++r) rows.push_back((int32_t)s->sub_worker[gr.subrows[r]]);
+        emit((int32_t)(b - a),
+             {Link{s->kv_indptr[rep], t0, std::min(len, t0 + per), qref, VA_NO_CAUSAL, lflags}},
+             std::move(rows));
+      }
+    }
+  }
+
+  // chains are split only when tiles alone cannot fill the machine
+  int32_t chain_split = 1;
+  if (chain_tiles > 0) {
+    const int64_t want = std::max<int64_t>(1, target - (int64_t)out.items.size());
+    if (chain_tiles < want) {
+      const int64_t avg = chain_tokens / chain_tiles;
+      chain_split = (int32_t)std::min<int64_t>((want + chain_tiles - 1) / chain_tiles,
+                                               std::max<int64_t>(1, avg / (8 * gran)));
+    }
+  }
+  for (auto& ch : chains) {
+    const int32_t nq = s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]];
+    for (int32_t a = 0; a < nq; a += q_tile) {
+      const int32_t b = std::min(nq, a + q_tile);
+      std::vector<Link> all;
+      int64_t tile_tokens = 0;
+      for (int32_t m : ch) {
+        const bool causal = s->flags[m] & VA_SUB_CAUSAL;
+        const int32_t len = s->seq_lens[m];
+        const int32_t vis = visible_end(len, nq, causal, b);
+        if (vis <= 0) continue;
+        const int32_t cbase = causal ? len - nq + a : VA_NO_CAUSAL;
+        all.push_back(Link{s->kv_indptr[m], 0, vis, s->qo_indptr[m] + a, cbase,
+                           (s->flags[m] & VA_SUB_SLOTS) ? VA_LINK_SLOTS : 0});
+        tile_tokens += vis;
+      }
+      std::vector<int32_t> rows;
+      for (int32_t r = a; r < b; ++r) rows.push_back((int32_t)s->sub_worker[s->qo_indptr[ch[0]] + r]);
+      if (all.empty()) continue;
+      const int32_t parts = (int32_t)std::max<int64_t>(1, std::min<int64_t>(chain_split, tile_tokens / (4 * gran)));
+      if (parts == 1) {
+        emit(b - a, all, std::move(rows));
+        continue;
+      }
+      const int32_t per = round_up((tile_tokens + parts - 1) / parts, gran);
+      std::vector<Link> cur;
+      int32_t room = per;
+      for (auto l : all) {
+        while (l.tok_begin < l.tok_end) {
+          const int32_t take = std::min(room, l.tok_end - l.tok_begin);
+          Link piece = l;
+          piece.tok_end = l.tok_begin + take;
+          cur.push_back(piece);
+          l.tok_begin += take;
+          room -= take;
+          if (room == 0) {
+            emit(b - a, cur, std::vector<int32_t>(rows));
+            cur.clear();
+            room = per;
+          }
+        }
+      }
+      if (!cur.empty()) emit(b - a, cur, std::vector<int32_t>(rows));
+    }
+  }
+
+  // ---- partial slots and the per-row merge lists ----
+  std::vector<std::vector<int32_t>> parts_of_row(s->n_rows);
+  for (auto& p : pend) {
+    bool direct = true;
+    for (int32_t r : p.rows) direct = direct && row_count[r] == 1;
+    Item& it = out.items[p.item];
+    if (direct) {
+      it.part_base = -1;
+    } else {
+      it.part_base = out.n_partials;
+      for (size_t i = 0; i < p.rows.size(); ++i) parts_of_row[p.rows[i]].push_back(out.n_partials + (int32_t)i);
+      out.n_partials += (int32_t)p.rows.size();
+    }
+  }
+  out.row_indptr.assign(s->n_rows + 1, 0);
+  out.row_flags.assign(s->n_rows, 0);
+  for (int32_t r = 0; r < s->n_rows; ++r) {
+    out.row_indptr[r + 1] = out.row_indptr[r] + (int32_t)parts_of_row[r].size();
+    out.row_ids.insert(out.row_ids.end(), parts_of_row[r].begin(), parts_of_row[r].end());
+    if (row_count[r] == 0) out.row_flags[r] = VA_ROW_EMPTY;
+    else if (parts_of_row[r].empty()) out.row_flags[r] = VA_ROW_DIRECT;
+  }
+
+  // longest items first: the tail of the launch is made of short items
+  std::vector<int32_t> order(out.items.size());
+  std::iota(order.begin(), order.end(), 0);
+  std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) {
+    return (int64_t)out.items[x].tokens * out.items[x].n_q > (int64_t)out.items[y].tokens * out.items[y].n_q;
+  });
+  std::vector<Item> sorted;
+  sorted.reserve(order.size());
+  for (int32_t i : order) sorted.push_back(out.items[i]);
+  out.items.swap(sorted);
+  return VA_OK;
+}
+
+void fill_counts(const Built& b, const VaSubRequests* s, const VaShape* shape, VaPlanCounts* c) {
+  c->kernel = b.kernel;
+  c->q_tile = b.q_tile;
+  c->kv_chunk = b.kv_chunk;
+  c->n_items = (int32_t)b.items.size();
+  c->n_links = (int32_t)b.links.size();
+  c->n_qrefs = (int32_t)b.qrefs.size();
+  c->n_partials = b.n_partials;
+  c->n_row_parts = (int32_t)b.row_ids.size();
+  c->plan_words = VA_PLAN_HEADER_WORDS + c->n_items * VA_ITEM_WORDS + c->n_links * VA_LINK_WORDS +
+                  c->n_qrefs + (s->n_rows + 1) + c->n_row_parts + s->n_rows;
+  c->workspace_bytes = va_workspace_bytes_for(b.n_partials, shape->num_q_heads, shape->head_dim);
+}
+
+}  // namespace
+
+extern "C" int va_plan_count(const VaSubRequests* subs, const VaShape* shape, const VaPlanParams* params,
+                             VaPlanCounts* counts) {
+  if (!counts) return va_fail(VA_ERR_ARG, "null counts");
+  Built b;
+  int rc = build(subs, shape, params, b);
+  if (rc) return rc;
+  fill_counts(b, subs, shape, counts);
+  return VA_OK;
+}
+
+extern "C" int va_plan_build(const VaSubRequests* subs, const VaShape* shape, const VaPlanParams* params,
+                             int32_t* plan_host, int64_t plan_capacity_words, VaPlanCounts* counts) {
+  if (!plan_host) return va_fail(VA_ERR_ARG, "null plan buffer");
+  Built b;
+  int rc = build(subs, shape, params, b);
+  if (rc) return rc;
+  VaPlanCounts c;
+  fill_counts(b, subs, shape, &c);
+  if (plan_capacity_words < c.plan_words)
+    return va_fail(VA_ERR_CAPACITY, "plan needs %d words, buffer holds %lld", c.plan_words,
+                   (long long)plan_capacity_words);
+  int32_t* h = plan_host;
+  int32_t off = VA_PLAN_HEADER_WORDS;
+  std::memset(h, 0, sizeof(int32_t) * VA_PLAN_HEADER_WORDS);
+  h[VA_H_MAGIC] = VA_PLAN_MAGIC;
+  h[VA_H_KERNEL] = c.kernel;
+  h[VA_H_Q_TILE] = c.q_tile;
+  h[VA_H_KV_CHUNK] = c.kv_chunk;
+  h[VA_H_N_ITEMS] = c.n_items;
+  h[VA_H_N_LINKS] = c.n_links;
+  h[VA_H_N_QREFS] = c.n_qrefs;
+  h[VA_H_N_PARTIALS] = c.n_partials;
+  h[VA_H_N_ROW_PARTS] = c.n_row_parts;
+  h[VA_H_N_ROWS] = subs->n_rows;
+  h[VA_H_N_SUBROWS] = subs->n_subrows;
+  h[VA_H_N_EMPTY_ROWS] = (int32_t)std::count(b.row_flags.begin(), b.row_flags.end(), VA_ROW_EMPTY);
+  h[VA_H_OFF_ITEMS] = off;
+  for (auto& it : b.items) {
+    int32_t* w = plan_host + off;
+    std::memset(w, 0, sizeof(int32_t) * VA_ITEM_WORDS);
+    w[VA_I_LINK_BEGIN] = it.link_begin;
+    w[VA_I_N_LINKS] = it.n_links;
+    w[VA_I_N_Q] = it.n_q;
+    w[VA_I_PART_BASE] = it.part_base;
+    w[VA_I_TOKENS] = it.tokens;
+    off += VA_ITEM_WORDS;
+  }
+  h[VA_H_OFF_LINKS] = off;
+  for (auto& l : b.links) {
+    int32_t* w = plan_host + off;
+    std::memset(w, 0, sizeof(int32_t) * VA_LINK_WORDS);
+    w[VA_L_KV_BEGIN] = l.kv_begin;
+    w[VA_L_TOK_BEGIN] = l.tok_begin;
+    w[VA_L_TOK_END] = l.tok_end;
+    w[VA_L_QREF] = l.qref;
+    w[VA_L_CAUSAL_BASE] = l.causal_base;
+    w[VA_L_FLAGS] = l.flags;
+    off += VA_LINK_WORDS;
+  }
+  h[VA_H_OFF_QREFS] = off;
+  std::copy(b.qrefs.begin(), b.qrefs.end(), plan_host + off);
+  off += c.n_qrefs;
+  h[VA_H_OFF_ROW_INDPTR] = off;
+  std::copy(b.row_indptr.begin(), b.row_indptr.end(), plan_host + off);
+  off += subs->n_rows + 1;
+  h[VA_H_OFF_ROW_IDS] = off;
+  std::copy(b.row_ids.begin(), b.row_ids.end(), plan_host + off);
+  off += c.n_row_parts;
+  h[VA_H_OFF_ROW_FLAGS] = off;
+  std::copy(b.row_flags.begin(), b.row_flags.end(), plan_host + off);
+  off += subs->n_rows;
+  if (counts) *counts = c;
+  return VA_OK;
+}

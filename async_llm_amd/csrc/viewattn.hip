@@ -1,0 +1,514 @@
+// libviewattn.so: C ABI, rotation/store kernel, vector-ALU attention kernel and
+// the partial-state merge kernel.  The matrix-core kernels live in va_mfma.hip.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/viewattn.h"
+#include "va_device.h"
+#include "va_internal.h"
+#include "va_launch.h"
+#include "va_plan.h"
+
+// ---------------------------------------------------------------------------
+// errors
+// ---------------------------------------------------------------------------
+static thread_local char g_error[512] = "";
+
+int va_fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+extern "C" const char* va_last_error(void) { return g_error; }
+extern "C" int va_version(void) { return 1; }
+
+int64_t va_workspace_bytes_for(int64_t n_partials, int num_q_heads, int head_dim) {
+  // accumulators [n_partials, Hq, D] fp32, then (max, sum) [n_partials, Hq, 2] fp32
+  return n_partials * num_q_heads * ((int64_t)head_dim + 2) * (int64_t)sizeof(float);
+}
+
+static int check_hip(hipError_t e, const char* what) {
+  if (e == hipSuccess) return VA_OK;
+  return va_fail(VA_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+namespace va {
+
+int make_rope(const VaRope* rope, int head_dim, RopeDev* out) {
+  if (!rope) return va_fail(VA_ERR_ARG, "null rope description");
+  if (rope->rotary_dim < 0 || rope->rotary_dim > head_dim || (rope->rotary_dim & 1))
+    return va_fail(VA_ERR_ARG, "rotary_dim %d must be even and within head_dim %d", rope->rotary_dim, head_dim);
+  out->mode = rope->mode;
+  out->rotary_dim = rope->rotary_dim;
+  out->half = rope->rotary_dim / 2;
+  out->cos_sin = rope->cos_sin_dev;
+  out->max_pos = rope->max_pos;
+  out->section_h3 = 3 * rope->section_h;
+  out->section_w3 = 3 * rope->section_w;
+  out->inv_freq = rope->inv_freq_dev;
+  if (rope->rotary_dim == 0) return VA_OK;
+  if (rope->mode == VA_ROPE_TABLE) {
+    if (!rope->cos_sin_dev || rope->max_pos <= 0) return va_fail(VA_ERR_ARG, "table rotation needs cos_sin and max_pos > 0");
+  } else if (rope->mode == VA_ROPE_MROPE) {
+    if (!rope->inv_freq_dev) return va_fail(VA_ERR_ARG, "mRoPE rotation needs inv_freq");
+  } else {
+    return va_fail(VA_ERR_ARG, "unknown rotation mode %d", rope->mode);
+  }
+  return VA_OK;
+}
+
+// ---------------------------------------------------------------------------
+// rotate (+ optional scatter of K and V rows into the pool)
+// ---------------------------------------------------------------------------
+// One workgroup per input row.  The row's heads are rotated pairwise
+// (i, i + rotary_dim/2) so the operation is safe in place; dims beyond
+// rotary_dim pass through.  With a destination table the rotated row goes to
+// pool row dst[i] (negative: the row is skipped, reference store.cu:44-46) and
+// the value row is copied beside it.
+template <typename E>
+__global__ __launch_bounds__(256) void rope_store_kernel(
+    const typename E::storage* __restrict__ x, const typename E::storage* __restrict__ v,
+    typename E::storage* y, typename E::storage* v_out, long long x_stride, long long v_stride,
+    long long y_stride, const void* dst, int dst_is_i64, const int64_t* pos, long long pos_axis_stride,
+    long long n_rows, int n_heads, int head_dim, RopeDev rope) {
+  const long long row = blockIdx.x;
+  if (row >= n_rows) return;
+  long long out_row = row;
+  if (dst) {
+    out_row = dst_is_i64 ? ((const long long*)dst)[row] : (long long)((const int*)dst)[row];
+    if (out_row < 0) return;
+  }
+  const typename E::storage* xr = x + row * x_stride;
+  typename E::storage* yr = y + out_row * y_stride;
+  const int half = rope.half;
+  if (half > 0) {
+    const Pos3 p = load_pos(pos, pos_axis_stride, row);
+    for (int e = threadIdx.x; e < n_heads * half; e += blockDim.x) {
+      const int h = e / half, i = e - h * half;
+      float c, s;
+      rope_cos_sin(rope, p, i, c, s);
+      const float x1 = E::load(xr[h * head_dim + i]);
+      const float x2 = E::load(xr[h * head_dim + half + i]);
+      float y1, y2;
+      rope_pair<E>(rope, c, s, x1, x2, y1, y2);
+      yr[h * head_dim + i] = E::store(y1);
+      yr[h * head_dim + half + i] = E::store(y2);
+    }
+  }
+  const int tail = head_dim - rope.rotary_dim;
+  if (tail > 0 && (const void*)xr != (const void*)yr) {
+    for (int e = threadIdx.x; e < n_heads * tail; e += blockDim.x) {
+      const int h = e / tail, i = e - h * tail;
+      yr[h * head_dim + rope.rotary_dim + i] = xr[h * head_dim + rope.rotary_dim + i];
+    }
+  }
+  if (v) {
+    const typename E::storage* vr = v + row * v_stride;
+    typename E::storage* vo = v_out + out_row * y_stride;
+    for (int e = threadIdx.x; e < n_heads * head_dim; e += blockDim.x) vo[e] = vr[e];
+  }
+}
+
+template <typename E>
+int launch_rope_store(const void* x, const void* v, void* y, void* v_out, long long x_stride,
+                      long long v_stride, long long y_stride, const void* dst, int dst_is_i64,
+                      const int64_t* pos, long long pos_axis_stride, long long n_rows, int n_heads,
+                      int head_dim, const RopeDev& rope, hipStream_t stream) {
+  using S = typename E::storage;
+  if (n_rows == 0) return VA_OK;
+  if (n_rows > 0x7fffffffLL) return va_fail(VA_ERR_ARG, "too many rows");
+  hipLaunchKernelGGL(rope_store_kernel<E>, dim3((unsigned)n_rows), dim3(256), 0, stream, (const S*)x,
+                     (const S*)v, (S*)y, (S*)v_out, x_stride, v_stride, y_stride, dst, dst_is_i64, pos,
+                     pos_axis_stride, n_rows, n_heads, head_dim, rope);
+  return check_hip(hipGetLastError(), "rope/store launch");
+}
+
+// ---------------------------------------------------------------------------
+// vector-ALU attention: any element type, head_dim in {16..256} (power of two)
+// ---------------------------------------------------------------------------
+// One workgroup (4 waves) per (work item, kv head).  Tile rows are taken one
+// after the other; for each, heads are processed in blocks of kHB.  A token's
+// K (then V) row is read by kLPT adjacent lanes with 16-byte loads, so a wave
+// streams 64/kLPT tokens per step and the four waves interleave tokens.  Every
+// lane group keeps its own online-softmax state; states are merged across lane
+// groups by shuffles and across waves through LDS when the chain ends.
+constexpr int kHB = 4;          // q heads per pass
+constexpr int kGenThreads = 256;
+constexpr int kGenWaves = kGenThreads / kWave;
+
+template <typename E, int kD>
+__global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
+  using S = typename E::storage;
+  constexpr int kVec = 16 / sizeof(S);
+  constexpr int kLPT = kD / kVec;  // lanes per token
+  constexpr int kTPW = kWave / kLPT;
+  static_assert(kLPT >= 1 && kLPT <= kWave, "head_dim out of range for this element type");
+
+  __shared__ float q_s[kHB][kD];
+  __shared__ float acc_s[kGenWaves][kHB][kD];
+  __shared__ float ml_s[kGenWaves][kHB][2];
+
+  const int32_t* item = a.items + (long long)blockIdx.x * VA_ITEM_WORDS;
+  const int hk = blockIdx.y;
+  const int G = a.num_q_heads / a.num_kv_heads;
+  const int n_q = item[VA_I_N_Q];
+  const int part_base = item[VA_I_PART_BASE];
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int li = lane % kLPT;   // which 16-byte piece of the row
+  const int lg = lane / kLPT;   // token within the wave step
+  const S* kp = (const S*)a.k_pool;
+  const S* vp = (const S*)a.v_pool;
+
+  for (int iq = 0; iq < n_q; ++iq) {
+    long long out_row = -1;
+    for (int hb = 0; hb < G; hb += kHB) {
+      float m[kHB], l[kHB], acc[kHB][kVec];
+#pragma unroll
+      for (int g = 0; g < kHB; ++g) {
+        m[g] = kNegBig;
+        l[g] = 0.f;
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) acc[g][e] = 0.f;
+      }
+      for (int li_ = 0; li_ < item[VA_I_N_LINKS]; ++li_) {
+        const int32_t* link = a.links + (long long)(item[VA_I_LINK_BEGIN] + li_) * VA_LINK_WORDS;
+        const int lflags = link[VA_L_FLAGS];
+        const int subrow = (lflags & VA_LINK_INDIRECT) ? a.qrefs[link[VA_L_QREF] + iq] : link[VA_L_QREF] + iq;
+        const long long src_row = a.sub_worker[subrow];
+        out_row = src_row;
+        const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
+
+        // rotate this row's query for the link, rounded to the element type
+        __syncthreads();
+        for (int e = threadIdx.x; e < kHB * kD; e += kGenThreads) {
+          const int g = e / kD, d = e - g * kD;
+          float val = 0.f;
+          if (hb + g < G) {
+            const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + hb + g) * kD;
+            if (d < a.rope.rotary_dim) {
+              const int i = d < a.rope.half ? d : d - a.rope.half;
+              float c, s;
+              rope_cos_sin(a.rope, p, i, c, s);
+              float y1, y2;
+              rope_pair<E>(a.rope, c, s, E::load(qh[i]), E::load(qh[i + a.rope.half]), y1, y2);
+              val = d < a.rope.half ? y1 : y2;
+            } else {
+              val = E::load(qh[d]);
+            }
+          }
+          q_s[g][d] = val;
+        }
+        __syncthreads();
+        float qr[kHB][kVec];
+#pragma unroll
+        for (int g = 0; g < kHB; ++g)
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) qr[g][e] = q_s[g][li * kVec + e];
+
+        const int t_end = min(link[VA_L_TOK_END], link[VA_L_CAUSAL_BASE] + iq + 1);
+        const int kv_begin = link[VA_L_KV_BEGIN];
+        const bool slots = lflags & VA_LINK_SLOTS;
+        for (int t0 = link[VA_L_TOK_BEGIN] + wave * kTPW; t0 < t_end; t0 += kGenWaves * kTPW) {
+          const int t = t0 + lg;
+          const bool live = t < t_end;
+          float sc[kHB];
+          uint4 kraw = make_uint4(0, 0, 0, 0), vraw = make_uint4(0, 0, 0, 0);
+          if (live) {
+            const long long slot = kv_slot(a.kv_indices, kv_begin, t, a.page_size, slots);
+            const long long off = slot * a.pool_row_stride + (long long)hk * kD + li * kVec;
+            kraw = *(const uint4*)(kp + off);
+            vraw = *(const uint4*)(vp + off);
+          }
+          const S* ke = (const S*)&kraw;
+          const S* ve = (const S*)&vraw;
+          float kf[kVec], vf[kVec];
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            kf[e] = E::load(ke[e]);
+            vf[e] = E::load(ve[e]);
+          }
+#pragma unroll
+          for (int g = 0; g < kHB; ++g) {
+            float d = 0.f;
+#pragma unroll
+            for (int e = 0; e < kVec; ++e) d = fmaf(qr[g][e], kf[e], d);
+            d = group_sum<kLPT>(d);
+            sc[g] = live ? d * a.scale_log2 : -INFINITY;
+          }
+#pragma unroll
+          for (int g = 0; g < kHB; ++g) {
+            const float m_new = fmaxf(m[g], sc[g]);
+            const float alpha = exp2f(m[g] - m_new);
+            const float pr = exp2f(sc[g] - m_new);
+            m[g] = m_new;
+            l[g] = l[g] * alpha + pr;
+#pragma unroll
+            for (int e = 0; e < kVec; ++e) acc[g][e] = fmaf(pr, vf[e], acc[g][e] * alpha);
+          }
+        }
+      }
+
+      // merge the lane groups of the wave
+#pragma unroll
+      for (int off = kLPT; off < kWave; off <<= 1) {
+#pragma unroll
+        for (int g = 0; g < kHB; ++g) {
+          const float m_o = __shfl_xor(m[g], off, kWave);
+          const float l_o = __shfl_xor(l[g], off, kWave);
+          const float m_new = fmaxf(m[g], m_o);
+          const float sa = exp2f(m[g] - m_new), sb = exp2f(m_o - m_new);
+          l[g] = l[g] * sa + l_o * sb;
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            const float a_o = __shfl_xor(acc[g][e], off, kWave);
+            acc[g][e] = acc[g][e] * sa + a_o * sb;
+          }
+          m[g] = m_new;
+        }
+      }
+      __syncthreads();
+      if (lg == 0) {
+#pragma unroll
+        for (int g = 0; g < kHB; ++g) {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) acc_s[wave][g][li * kVec + e] = acc[g][e];
+          if (li == 0) {
+            ml_s[wave][g][0] = m[g];
+            ml_s[wave][g][1] = l[g];
+          }
+        }
+      }
+      __syncthreads();
+      // merge the waves and emit
+      for (int e = threadIdx.x; e < kHB * kD; e += kGenThreads) {
+        const int g = e / kD, d = e - g * kD;
+        if (hb + g >= G) continue;
+        float mm = kNegBig;
+#pragma unroll
+        for (int w = 0; w < kGenWaves; ++w) mm = fmaxf(mm, ml_s[w][g][0]);
+        float ll = 0.f, av = 0.f;
+#pragma unroll
+        for (int w = 0; w < kGenWaves; ++w) {
+          const float sw = exp2f(ml_s[w][g][0] - mm);
+          ll += ml_s[w][g][1] * sw;
+          av += acc_s[w][g][d] * sw;
+        }
+        const int hq = hk * G + hb + g;
+        if (part_base < 0) {
+          S* o = (S*)a.out + (out_row * a.num_q_heads + hq) * (long long)kD;
+          o[d] = E::store(ll > 0.f ? av / ll : 0.f);
+          if (d == 0 && a.lse) {
+            const float lse2 = ll > 0.f ? mm + log2f(ll) : -INFINITY;
+            a.lse[out_row * a.num_q_heads + hq] = a.lse_base2 ? lse2 : lse2 * kLn2;
+          }
+        } else {
+          const long long slot = (long long)(part_base + iq) * a.num_q_heads + hq;
+          a.part_acc[slot * kD + d] = av;
+          if (d == 0) {
+            a.part_ml[slot * 2 + 0] = mm;
+            a.part_ml[slot * 2 + 1] = ll;
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// merge of partial states: one workgroup of 64 lanes per (row, q head)
+// ---------------------------------------------------------------------------
+template <typename E>
+__global__ __launch_bounds__(64) void merge_kernel(MergeArgs a) {
+  using S = typename E::storage;
+  const long long row = blockIdx.x;
+  const int hq = blockIdx.y;
+  const int flags = a.row_flags[row];
+  if (flags & VA_ROW_DIRECT) return;
+  S* o = (S*)a.out + (row * a.num_q_heads + hq) * (long long)a.head_dim;
+  if (flags & VA_ROW_EMPTY) {
+    for (int d = threadIdx.x; d < a.head_dim; d += 64) o[d] = E::store(0.f);
+    if (threadIdx.x == 0 && a.lse) a.lse[row * a.num_q_heads + hq] = -INFINITY;
+    return;
+  }
+  const int b = a.row_indptr[row], e = a.row_indptr[row + 1];
+  float mm = kNegBig;
+  for (int i = b; i < e; ++i) mm = fmaxf(mm, a.part_ml[((long long)a.row_ids[i] * a.num_q_heads + hq) * 2]);
+  float ll = 0.f;
+  for (int i = b; i < e; ++i) {
+    const long long slot = (long long)a.row_ids[i] * a.num_q_heads + hq;
+    ll += a.part_ml[slot * 2 + 1] * exp2f(a.part_ml[slot * 2] - mm);
+  }
+  for (int d = threadIdx.x; d < a.head_dim; d += 64) {
+    float av = 0.f;
+    for (int i = b; i < e; ++i) {
+      const long long slot = (long long)a.row_ids[i] * a.num_q_heads + hq;
+      av += a.part_acc[slot * a.head_dim + d] * exp2f(a.part_ml[slot * 2] - mm);
+    }
+    o[d] = E::store(ll > 0.f ? av / ll : 0.f);
+  }
+  if (threadIdx.x == 0 && a.lse) {
+    const float lse2 = ll > 0.f ? mm + log2f(ll) : -INFINITY;
+    a.lse[row * a.num_q_heads + hq] = a.lse_base2 ? lse2 : lse2 * kLn2;
+  }
+}
+
+template <typename E>
+int launch_generic(const AttnArgs& a, int n_items, hipStream_t stream) {
+  const dim3 grid((unsigned)n_items, (unsigned)a.num_kv_heads), block(kGenThreads);
+  constexpr int kMaxD = 16 / sizeof(typename E::storage) * 64;
+  switch (a.head_dim) {
+#define VA_CASE(D)                                                              \
+  case D:                                                                       \
+    if constexpr (D <= kMaxD && D >= 16 / (int)sizeof(typename E::storage)) {   \
+      hipLaunchKernelGGL((attn_generic_kernel<E, D>), grid, block, 0, stream, a); \
+      break;                                                                    \
+    }                                                                           \
+    return va_fail(VA_ERR_ARG, "head_dim %d unsupported for this element type", a.head_dim);
+    VA_CASE(16)
+    VA_CASE(32)
+    VA_CASE(64)
+    VA_CASE(128)
+    VA_CASE(256)
+#undef VA_CASE
+    default:
+      return va_fail(VA_ERR_ARG, "head_dim %d unsupported (16, 32, 64, 128 or 256)", a.head_dim);
+  }
+  return check_hip(hipGetLastError(), "attention launch");
+}
+
+template <typename E>
+int launch_merge(const MergeArgs& a, int n_rows, hipStream_t stream) {
+  hipLaunchKernelGGL(merge_kernel<E>, dim3((unsigned)n_rows, (unsigned)a.num_q_heads), dim3(64), 0, stream, a);
+  return check_hip(hipGetLastError(), "merge launch");
+}
+
+}  // namespace va
+
+// ---------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------
+#define VA_DISPATCH_DTYPE(dtype, CALL)                                  \
+  switch (dtype) {                                                      \
+    case VA_F32: { using E = va::F32; CALL; } break;                    \
+    case VA_F16: { using E = va::F16; CALL; } break;                    \
+    case VA_BF16: { using E = va::BF16; CALL; } break;                  \
+    default: return va_fail(VA_ERR_ARG, "unknown dtype %d", (int)(dtype)); \
+  }
+
+extern "C" int va_rope(const void* x_dev, void* y_dev, const int64_t* pos_dev, int64_t pos_axis_stride,
+                       int64_t n_rows, int32_t n_heads, int32_t head_dim, int32_t dtype,
+                       int64_t x_row_stride, int64_t y_row_stride, const VaRope* rope, void* stream) {
+  if (n_rows < 0 || n_heads <= 0 || head_dim <= 0) return va_fail(VA_ERR_ARG, "bad shape");
+  if (n_rows == 0) return VA_OK;
+  if (!x_dev || !y_dev || !pos_dev) return va_fail(VA_ERR_ARG, "null pointer");
+  va::RopeDev r;
+  int rc = va::make_rope(rope, head_dim, &r);
+  if (rc) return rc;
+  VA_DISPATCH_DTYPE(dtype, rc = va::launch_rope_store<E>(x_dev, nullptr, y_dev, nullptr, x_row_stride, 0,
+                                                         y_row_stride, nullptr, 0, pos_dev, pos_axis_stride,
+                                                         n_rows, n_heads, head_dim, r, (hipStream_t)stream));
+  return rc;
+}
+
+extern "C" int va_store_kv_rope(const void* k_dev, const void* v_dev, int64_t k_row_stride,
+                                int64_t v_row_stride, void* k_pool_dev, void* v_pool_dev,
+                                int64_t pool_row_stride, const void* out_loc_dev, int32_t out_loc_is_i64,
+                                const int64_t* pos_dev, int64_t pos_axis_stride, int64_t n_rows,
+                                const VaShape* shape, const VaRope* rope, void* stream) {
+  if (!shape) return va_fail(VA_ERR_ARG, "null shape");
+  if (n_rows < 0) return va_fail(VA_ERR_ARG, "bad shape");
+  if (n_rows == 0) return VA_OK;
+  if (!k_dev || !v_dev || !k_pool_dev || !v_pool_dev || !out_loc_dev || !pos_dev)
+    return va_fail(VA_ERR_ARG, "null pointer");
+  va::RopeDev r;
+  int rc = va::make_rope(rope, shape->head_dim, &r);
+  if (rc) return rc;
+  VA_DISPATCH_DTYPE(shape->dtype,
+                    rc = va::launch_rope_store<E>(k_dev, v_dev, k_pool_dev, v_pool_dev, k_row_stride, v_row_stride,
+                                                  pool_row_stride, out_loc_dev, out_loc_is_i64, pos_dev,
+                                                  pos_axis_stride, n_rows, shape->num_kv_heads, shape->head_dim, r,
+                                                  (hipStream_t)stream));
+  return rc;
+}
+
+extern "C" int va_attention(const void* q_dev, int64_t q_row_stride, const void* k_pool_dev,
+                            const void* v_pool_dev, int64_t pool_row_stride, const int32_t* plan_dev,
+                            const int32_t* plan_header_host, const int32_t* kv_indices_dev,
+                            const int64_t* sub_worker_dev, const int64_t* sub_loc_dev,
+                            int64_t sub_loc_axis_stride, void* out_dev, float* lse_dev, int32_t lse_base2,
+                            void* workspace_dev, int64_t workspace_bytes, const VaShape* shape,
+                            const VaRope* rope, void* stream) {
+  if (!shape || !plan_header_host || !plan_dev) return va_fail(VA_ERR_ARG, "null plan or shape");
+  const int32_t* h = plan_header_host;
+  if (h[VA_H_MAGIC] != VA_PLAN_MAGIC) return va_fail(VA_ERR_ARG, "plan header has no magic word");
+  const int n_rows = h[VA_H_N_ROWS], n_items = h[VA_H_N_ITEMS], n_partials = h[VA_H_N_PARTIALS];
+  if (n_rows == 0) return VA_OK;
+  if (!out_dev) return va_fail(VA_ERR_ARG, "null out");
+  if (n_items > 0 && (!q_dev || !k_pool_dev || !v_pool_dev || !sub_worker_dev || !sub_loc_dev || !kv_indices_dev))
+    return va_fail(VA_ERR_ARG, "null pointer");
+  if (shape->num_kv_heads <= 0 || shape->num_q_heads % shape->num_kv_heads)
+    return va_fail(VA_ERR_ARG, "num_q_heads must be a multiple of num_kv_heads");
+  const int64_t need = va_workspace_bytes_for(n_partials, shape->num_q_heads, shape->head_dim);
+  if (need > 0 && (!workspace_dev || workspace_bytes < need))
+    return va_fail(VA_ERR_CAPACITY, "workspace needs %lld bytes, got %lld", (long long)need, (long long)workspace_bytes);
+  va::RopeDev r;
+  int rc = va::make_rope(rope, shape->head_dim, &r);
+  if (rc) return rc;
+
+  va::AttnArgs a;
+  a.q = q_dev;
+  a.q_row_stride = q_row_stride;
+  a.k_pool = k_pool_dev;
+  a.v_pool = v_pool_dev;
+  a.pool_row_stride = pool_row_stride;
+  a.items = plan_dev + h[VA_H_OFF_ITEMS];
+  a.links = plan_dev + h[VA_H_OFF_LINKS];
+  a.qrefs = plan_dev + h[VA_H_OFF_QREFS];
+  a.kv_indices = kv_indices_dev;
+  a.sub_worker = sub_worker_dev;
+  a.sub_loc = sub_loc_dev;
+  a.sub_loc_axis_stride = sub_loc_axis_stride;
+  a.out = out_dev;
+  a.lse = lse_dev;
+  a.lse_base2 = lse_base2;
+  a.part_acc = (float*)workspace_dev;
+  a.part_ml = (float*)workspace_dev + (int64_t)n_partials * shape->num_q_heads * shape->head_dim;
+  a.num_q_heads = shape->num_q_heads;
+  a.num_kv_heads = shape->num_kv_heads;
+  a.head_dim = shape->head_dim;
+  a.page_size = shape->page_size;
+  a.rope = r;
+  a.scale_log2 = va::kLog2e / sqrtf((float)shape->head_dim);
+  hipStream_t s = (hipStream_t)stream;
+
+  if (n_items > 0) {
+    if (h[VA_H_KERNEL] == VA_KERNEL_MFMA) {
+      rc = va::launch_mfma(a, shape->dtype, n_items, h[VA_H_Q_TILE], s);
+    } else {
+      VA_DISPATCH_DTYPE(shape->dtype, rc = va::launch_generic<E>(a, n_items, s));
+    }
+    if (rc) return rc;
+  }
+  if (n_partials > 0 || h[VA_H_N_EMPTY_ROWS] > 0) {
+    va::MergeArgs m;
+    m.row_indptr = plan_dev + h[VA_H_OFF_ROW_INDPTR];
+    m.row_ids = plan_dev + h[VA_H_OFF_ROW_IDS];
+    m.row_flags = plan_dev + h[VA_H_OFF_ROW_FLAGS];
+    m.part_acc = a.part_acc;
+    m.part_ml = a.part_ml;
+    m.out = out_dev;
+    m.lse = lse_dev;
+    m.lse_base2 = lse_base2;
+    m.num_q_heads = shape->num_q_heads;
+    m.head_dim = shape->head_dim;
+    VA_DISPATCH_DTYPE(shape->dtype, rc = va::launch_merge<E>(m, n_rows, s));
+  }
+  return rc;
+}

@@ -1,0 +1,197 @@
+/*
+ * viewattn.h -- C ABI of libviewattn.so: cache-view attention for MI355X (gfx950).
+ *
+ * The library replaces, for AsyncLLM's view-attention path, everything the
+ * reference hands to third-party CUDA code or to torch elementwise ops inside
+ * SharedCacheAttention.forward:
+ *
+ *   reference (python/minisgl/...)                          entry point here
+ *   ------------------------------------------------------  ------------------
+ *   shared_cache/rope_correction.py:15-54,                  va_rope
+ *     shared_cache/attention.py:241-280 (_rope/_rope_mrope)
+ *   attention.py:645-649 + kernel/store.py:30-42 +          va_store_kv_rope
+ *     kernel/csrc/jit/store.cu:27-125 (K rotate + KV store)
+ *   FlashInfer wrapper.plan(...) attention.py:390-426,      va_plan_count,
+ *     574-604 (work decomposition of the planned tables)    va_plan_build
+ *   attention.py:652-703 (q gather + per-segment rotate,    va_attention
+ *     BatchDecode run x2, pad-scatter, merge_states) and
+ *     attention.py:705-752 (BatchPrefill run x2, merge)
+ *
+ * Conventions: every function returns 0 on success or a negative VA_ERR_*;
+ * va_last_error() returns a thread-local message for the last failure.  All
+ * pointers named *_dev are device pointers on the current HIP device; *_host are
+ * host pointers.  The library allocates nothing and keeps no global state: the
+ * caller owns every buffer (workspace included) and the stream.  `stream` is a
+ * hipStream_t passed as void*.
+ */
+#ifndef VIEWATTN_H
+#define VIEWATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define VA_API __attribute__((visibility("default")))
+#else
+#define VA_API
+#endif
+
+#define VA_OK 0
+#define VA_ERR_ARG (-1)       /* inconsistent or unsupported argument */
+#define VA_ERR_CAPACITY (-2)  /* caller-provided buffer too small */
+#define VA_ERR_HIP (-3)       /* a HIP runtime call failed */
+
+/* element types of q/k/v/out and of the KV pool */
+#define VA_F32 0
+#define VA_F16 1
+#define VA_BF16 2
+
+/* rotation modes */
+#define VA_ROPE_TABLE 0 /* 1-D neox RoPE from an fp32 cos|sin table (rope_correction.py) */
+#define VA_ROPE_MROPE 1 /* interleaved 3-axis mRoPE, cos/sin computed from inv_freq      */
+
+/* kernel families for va_attention / va_plan_* */
+#define VA_KERNEL_AUTO 0
+#define VA_KERNEL_GENERIC 1 /* vector-ALU path, any dtype                            */
+#define VA_KERNEL_MFMA 2    /* bf16/f16 matrix-core path                             */
+
+typedef struct VaShape {
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t head_dim;
+  int32_t page_size; /* tokens per page of the pool */
+  int32_t dtype;     /* VA_F32 / VA_F16 / VA_BF16 */
+} VaShape;
+
+typedef struct VaRope {
+  int32_t mode;          /* VA_ROPE_TABLE / VA_ROPE_MROPE */
+  int32_t rotary_dim;    /* leading head dims that rotate (pairs i, i+rotary_dim/2) */
+  const float* cos_sin_dev; /* [max_pos, rotary_dim] fp32: cos | sin  (TABLE)       */
+  int32_t max_pos;       /* rows of the table; |position| is clamped to max_pos-1  */
+  int32_t section_h;     /* mrope_section[1] (MROPE)                                */
+  int32_t section_w;     /* mrope_section[2] (MROPE)                                */
+  const float* inv_freq_dev; /* [rotary_dim/2] fp32 (MROPE)                         */
+} VaRope;
+
+VA_API const char* va_last_error(void);
+VA_API int va_version(void);
+
+/*
+ * va_rope: y[i, h, :] = R(pos[i]) x[i, h, :] for i < n_rows, h < n_heads.
+ * pos_dev is int64 [n_rows] (pos_axis_stride == 0) or [3, n_rows] with
+ * pos_axis_stride elements between axes (mRoPE with genuine 3-D positions).
+ * x/y rows are x_row_stride / y_row_stride ELEMENTS apart; heads are
+ * contiguous (head_dim apart).  In-place (y == x) is allowed.
+ * Replaces rope_correction.py:15-54 and attention.py:241-280.
+ */
+VA_API int va_rope(const void* x_dev, void* y_dev, const int64_t* pos_dev, int64_t pos_axis_stride,
+            int64_t n_rows, int32_t n_heads, int32_t head_dim, int32_t dtype,
+            int64_t x_row_stride, int64_t y_row_stride, const VaRope* rope, void* stream);
+
+/*
+ * va_store_kv_rope: for every row i with out_loc[i] >= 0 write
+ *   k_pool[out_loc[i]] = R(pos[i]) k[i]   and   v_pool[out_loc[i]] = v[i]
+ * (rows with a negative slot are skipped: store.cu:44-46).  out_loc is int32 or
+ * int64 (out_loc_is_i64).  Pool rows are pool_row_stride elements apart and
+ * hold num_kv_heads*head_dim elements.  Replaces attention.py:645-649 +
+ * store.cu:27-57 in one pass (the rotated key is never materialised).
+ */
+VA_API int va_store_kv_rope(const void* k_dev, const void* v_dev, int64_t k_row_stride,
+                     int64_t v_row_stride, void* k_pool_dev, void* v_pool_dev,
+                     int64_t pool_row_stride, const void* out_loc_dev, int32_t out_loc_is_i64,
+                     const int64_t* pos_dev, int64_t pos_axis_stride, int64_t n_rows,
+                     const VaShape* shape, const VaRope* rope, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Work decomposition (host).  Input: the planned sub-request tables, exactly the
+ * integer tensors the reference hands to FlashInfer's plan():
+ *   sub-request s reads KV entries kv_indptr[s]..kv_indptr[s+1] of kv_indices
+ *   (page numbers, or token slots when VA_SUB_SLOTS is set: the page_size=1
+ *   aux wrapper of attention.py:412-426), seq_lens[s] tokens, and serves the
+ *   query sub-rows qo_indptr[s]..qo_indptr[s+1] (indices into sub_worker /
+ *   sub_loc).  flags[s]: VA_SUB_CAUSAL = bottom-right aligned causal mask
+ *   (attention.py:586-602).  chain[s] >= 0 ties the sub-requests of one prefill
+ *   request together (same query rows, merged in-kernel); chain[s] < 0 marks a
+ *   stand-alone (decode) sub-request, which may be batched with other
+ *   sub-requests that read the identical page list.
+ * ------------------------------------------------------------------------- */
+#define VA_SUB_CAUSAL 1
+#define VA_SUB_SLOTS 2
+
+typedef struct VaSubRequests {
+  int32_t n_sub;
+  int32_t n_subrows;          /* == qo_indptr[n_sub] */
+  int32_t n_rows;             /* output rows (workers / new tokens) */
+  const int32_t* qo_indptr;   /* [n_sub+1] host */
+  const int32_t* kv_indptr;   /* [n_sub+1] host */
+  const int32_t* kv_indices;  /* [kv_indptr[n_sub]] host */
+  const int32_t* seq_lens;    /* [n_sub] host */
+  const int32_t* flags;       /* [n_sub] host */
+  const int32_t* chain;       /* [n_sub] host */
+  const int64_t* sub_worker;  /* [n_subrows] host: output row of each sub-row */
+} VaSubRequests;
+
+typedef struct VaPlanParams {
+  int32_t kernel;        /* VA_KERNEL_*; AUTO picks by dtype/shape            */
+  int32_t q_tile;        /* 0 = library default for the chosen kernel         */
+  int32_t kv_chunk;      /* 0 = derive from the launch's total KV tokens      */
+  int32_t target_items;  /* 0 = default (work items wanted per kv head)       */
+} VaPlanParams;
+
+typedef struct VaPlanCounts {
+  int32_t kernel;        /* resolved kernel family */
+  int32_t q_tile;        /* resolved */
+  int32_t kv_chunk;      /* resolved */
+  int32_t n_items;
+  int32_t n_links;
+  int32_t n_qrefs;
+  int32_t n_partials;    /* partial (row, item) slots the launch will write */
+  int32_t n_row_parts;   /* length of row_part_ids */
+  int32_t plan_words;    /* int32 words va_plan_build writes                 */
+  int64_t workspace_bytes; /* device scratch va_attention needs for this plan */
+} VaPlanCounts;
+
+/* Size the plan (no output besides *counts). */
+VA_API int va_plan_count(const VaSubRequests* subs, const VaShape* shape, const VaPlanParams* params,
+                  VaPlanCounts* counts);
+
+/*
+ * Build the plan into plan_host (capacity plan_capacity_words int32 words, at
+ * least counts->plan_words).  The blob is position independent: copy it to the
+ * device verbatim and pass the device copy to va_attention.  Layout (int32
+ * words): header[24] | items[n_items*8] | links[n_links*8] | qrefs[n_qrefs] |
+ * row_part_indptr[n_rows+1] | row_part_ids[n_row_parts] | row_flags[n_rows].
+ */
+VA_API int va_plan_build(const VaSubRequests* subs, const VaShape* shape, const VaPlanParams* params,
+                  int32_t* plan_host, int64_t plan_capacity_words, VaPlanCounts* counts);
+
+/*
+ * va_attention: out[r, h, :] = softmax over the whole view of row r, i.e. the
+ * LSE merge over all sub-requests (and KV chunks) that serve row r of
+ *   softmax(R(sub_loc[i]) q[sub_worker[i], h] . K_s^T / sqrt(head_dim)) V_s .
+ * q is [n_q_rows, num_q_heads, head_dim] unrotated, rows q_row_stride elements
+ * apart; the pool is [num_slots, num_kv_heads, head_dim] with slot stride
+ * pool_row_stride elements; out is [n_rows, num_q_heads*head_dim] contiguous;
+ * lse_dev (optional, may be NULL) is fp32 [n_rows, num_q_heads]: natural-log
+ * logsumexp of the scaled scores, or log2 when lse_base2 != 0.
+ * sub_loc_dev is int64 [n_subrows] (sub_loc_axis_stride == 0) or [3, n_subrows].
+ * plan_dev / kv_indices_dev / sub_worker_dev are device copies of the host
+ * tables the plan was built from.  Rows no sub-request serves get out = 0 and
+ * lse = -inf.  workspace_dev must hold counts.workspace_bytes.
+ */
+VA_API int va_attention(const void* q_dev, int64_t q_row_stride, const void* k_pool_dev,
+                 const void* v_pool_dev, int64_t pool_row_stride, const int32_t* plan_dev,
+                 const int32_t* plan_header_host, const int32_t* kv_indices_dev,
+                 const int64_t* sub_worker_dev, const int64_t* sub_loc_dev,
+                 int64_t sub_loc_axis_stride, void* out_dev, float* lse_dev, int32_t lse_base2,
+                 void* workspace_dev, int64_t workspace_bytes, const VaShape* shape,
+                 const VaRope* rope, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VIEWATTN_H */
