@@ -75,6 +75,8 @@ __device__ __forceinline__ Pos3 load_pos(const int64_t* pos, int64_t axis_stride
   return p;
 }
 
+__device__ __forceinline__ float mul_rounded(float a, float b);
+
 // cos/sin of rotary pair `i` (0 <= i < half) at position `p`.
 //  TABLE: row |p| (clamped to the table) of the fp32 cos|sin cache, sine negated for
 //         negative p  (reference rope_correction.py:36-42).
@@ -82,7 +84,6 @@ __device__ __forceinline__ Pos3 load_pos(const int64_t* pos, int64_t axis_stride
 //         i % 3 == 1 and i < 3*section[1], the width axis when i % 3 == 2 and
 //         i < 3*section[2], the temporal axis otherwise  (reference attention.py:267-277).
 __device__ __forceinline__ void rope_cos_sin(const RopeDev& r, const Pos3& p, int i, float& c, float& s) {
-#pragma clang fp contract(off)
   if (r.mode == VA_ROPE_TABLE) {
     long long a = p.t < 0 ? -p.t : p.t;
     if (a > r.max_pos - 1) a = r.max_pos - 1;
@@ -95,7 +96,7 @@ __device__ __forceinline__ void rope_cos_sin(const RopeDev& r, const Pos3& p, in
     long long q = p.t;
     if (m == 1 && i < r.section_h3) q = p.h;
     if (m == 2 && i < r.section_w3) q = p.w;
-    const float angle = __fmul_rn((float)q, r.inv_freq[i]);
+    const float angle = mul_rounded((float)q, r.inv_freq[i]);
     c = cosf(angle);
     s = sinf(angle);
   }
@@ -106,17 +107,24 @@ __device__ __forceinline__ void rope_cos_sin(const RopeDev& r, const Pos3& p, in
 //  MROPE: cos/sin are first cast to the element type and every product and the sum
 //         are rounded to it, as torch does for `x*cos + rotate_half(x)*sin` on a
 //         low-precision tensor (attention.py:276-279).
+// A product that the compiler may not fuse into a following add (the reference
+// computes rotations with separately rounded multiplies and adds).
+__device__ __forceinline__ float mul_rounded(float a, float b) {
+  float p = a * b;
+  asm volatile("" : "+v"(p));
+  return p;
+}
+
 template <typename E>
 __device__ __forceinline__ void rope_pair(const RopeDev& r, float c, float s, float x1, float x2,
                                           float& y1, float& y2) {
-#pragma clang fp contract(off)
   if (r.mode == VA_ROPE_TABLE) {
-    y1 = round_through<E>(__fsub_rn(__fmul_rn(c, x1), __fmul_rn(s, x2)));
-    y2 = round_through<E>(__fadd_rn(__fmul_rn(c, x2), __fmul_rn(s, x1)));
+    y1 = round_through<E>(mul_rounded(c, x1) - mul_rounded(s, x2));
+    y2 = round_through<E>(mul_rounded(c, x2) + mul_rounded(s, x1));
   } else {
     const float ce = round_through<E>(c), se = round_through<E>(s);
-    y1 = round_through<E>(__fadd_rn(round_through<E>(__fmul_rn(x1, ce)), round_through<E>(__fmul_rn(-x2, se))));
-    y2 = round_through<E>(__fadd_rn(round_through<E>(__fmul_rn(x2, ce)), round_through<E>(__fmul_rn(x1, se))));
+    y1 = round_through<E>(round_through<E>(mul_rounded(x1, ce)) + round_through<E>(mul_rounded(-x2, se)));
+    y2 = round_through<E>(round_through<E>(mul_rounded(x2, ce)) + round_through<E>(mul_rounded(x1, se)));
   }
 }
 

@@ -425,8 +425,9 @@ extern "C" int va_store_kv_rope(const void* k_dev, const void* v_dev, int64_t k_
   if (!shape) return va_fail(VA_ERR_ARG, "null shape");
   if (n_rows < 0) return va_fail(VA_ERR_ARG, "bad shape");
   if (n_rows == 0) return VA_OK;
-  if (!k_dev || !v_dev || !k_pool_dev || !v_pool_dev || !out_loc_dev || !pos_dev)
+  if (!k_dev || !v_dev || !k_pool_dev || !v_pool_dev || !out_loc_dev || !rope)
     return va_fail(VA_ERR_ARG, "null pointer");
+  if (!pos_dev && rope->rotary_dim > 0) return va_fail(VA_ERR_ARG, "rotation needs positions");
   va::RopeDev r;
   int rc = va::make_rope(rope, shape->head_dim, &r);
   if (rc) return rc;

@@ -66,10 +66,9 @@ def store_rows(k_cache: torch.Tensor, v_cache: torch.Tensor, indices: torch.Tens
     n = k.shape[0]
     assert indices.dtype in (torch.int32, torch.int64) and indices.numel() == n
     indices = indices.contiguous()
-    zeros = torch.zeros(n, dtype=torch.int64, device=k.device)
     shape = native.make_shape(1, 1, width, 1, k.dtype)
     rope = native.VaRope(native.VA_ROPE_TABLE, 0, None, 0, 0, 0, None)
     native.check(native.lib.va_store_kv_rope(
         k.data_ptr(), v.data_ptr(), k.stride(0), v.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
-        k_cache.stride(0), indices.data_ptr(), int(indices.dtype == torch.int64), zeros.data_ptr(), 0,
+        k_cache.stride(0), indices.data_ptr(), int(indices.dtype == torch.int64), None, 0,
         n, shape, rope, native.current_stream_ptr(k.device)))

@@ -162,11 +162,15 @@ def make_rope(rotary_dim: int, cos_sin: Optional[torch.Tensor], inv_freq: Option
     (cos/sin from ``inv_freq``), else the 1-D fp32 cos|sin table."""
     if mrope_section is not None:
         assert inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.is_contiguous()
-        return VaRope(VA_ROPE_MROPE, rotary_dim, None, 0, int(mrope_section[1]), int(mrope_section[2]),
+        rope = VaRope(VA_ROPE_MROPE, rotary_dim, None, 0, int(mrope_section[1]), int(mrope_section[2]),
                       inv_freq.data_ptr())
+        rope._keepalive = inv_freq  # the struct only holds the raw device address
+        return rope
     assert cos_sin is not None
     if cos_sin.dtype != torch.float32 or not cos_sin.is_contiguous():
         raise ViewAttnError("cos_sin_cache must be a contiguous fp32 [max_pos, rotary_dim] tensor")
     if rotary_dim and cos_sin.shape[1] != rotary_dim:
         raise ViewAttnError(f"cos_sin_cache has {cos_sin.shape[1]} columns, rotary_dim is {rotary_dim}")
-    return VaRope(VA_ROPE_TABLE, rotary_dim, cos_sin.data_ptr(), cos_sin.shape[0], 0, 0, None)
+    rope = VaRope(VA_ROPE_TABLE, rotary_dim, cos_sin.data_ptr(), cos_sin.shape[0], 0, 0, None)
+    rope._keepalive = cos_sin
+    return rope

@@ -1,0 +1,221 @@
+"""Benchmark of cache-view attention on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload batched_decode]
+
+A step is one ``SharedCacheAttention.forward`` of one layer (fused key
+rotate + KV store, attention, merge) over the batched bf16 decode
+configuration: 64 requests, 16 q / 4 kv heads, head_dim 256, page size 16,
+every view = one shared 8192-token block + 1-3 private blocks of 256..8192
+tokens.  Inputs are resident in HBM before the timed region; successive steps
+rotate over several copies of the KV pool so the 256 MB last-level cache cannot
+hold the working set.  Prints ONE JSON line.
+
+``value`` is algorithmic GB/s: compulsory bytes of a step (each distinct block
+counted once, see ``async_llm_amd.workloads``) divided by the wall time per
+step.  ``roofline`` prices the attention kernel alone, timed with HIP events on
+the stream it is launched on.  ``cpu_baseline`` times the CPU oracle (torch on
+the host cores) on a bounded sample of the same workload.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default="batched_decode",
+                    choices=["batched_decode", "mrope_decode", "view_prefill", "plumbing_decode"])
+    ap.add_argument("--layers", type=int, default=4, help="copies of the KV pool rotated over")
+    ap.add_argument("--kernel", default=None, choices=[None, "auto", "generic", "mfma"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample", type=int, default=0, help="requests in the CPU sample (0 = pick by size)")
+    ap.add_argument("--extra", action="store_true", help="also time the prefill configuration")
+    return ap.parse_args()
+
+
+def build_workload(name, device, layers, kernel):
+    from async_llm_amd import workloads
+
+    if name == "batched_decode":
+        return workloads.batched_decode(device, layers=layers, kernel=kernel)
+    if name == "mrope_decode":
+        return workloads.mrope_decode(device, layers=layers, kernel=kernel)
+    if name == "view_prefill":
+        return workloads.view_prefill(device, layers=layers, kernel=kernel)
+    return workloads.plumbing_decode(device, layers=layers, kernel=kernel)
+
+
+def time_attention_kernel(wl, steps, warmup, layers):
+    """Average duration of the attention launch alone (store excluded), HIP
+    events recorded on the stream the kernels run on."""
+    import torch
+
+    op, meta = wl.op, wl.meta
+    stream = torch.cuda.current_stream()
+    for i in range(warmup):
+        op.attend(wl.q, i % layers, meta)
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    for i in range(steps):
+        starts[i].record(stream)
+        op.attend(wl.q, i % layers, meta)
+        stops[i].record(stream)
+    torch.cuda.synchronize()
+    times = sorted(s.elapsed_time(e) for s, e in zip(starts, stops))
+    return sum(times) / len(times), times[len(times) // 2]
+
+
+def cpu_baseline(wl, sample):
+    """The CPU oracle on the first ``sample`` requests of the workload (same
+    blocks, same inputs): rotate+store, per-segment attention, merge."""
+    import torch
+
+    from async_llm_amd.shared_cache import WorkerGroup
+    from oracle import view_attention_oracle as O
+    from tests.util import oracle_decode_plan, oracle_prefill_plan, oracle_rope
+
+    op = wl.op
+    Hq, Hkv, D, P = op.num_qo_heads, op.num_kv_heads, op.head_dim, op.page_size
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    rope = oracle_rope(op, wl.theta)
+    k_cpu, v_cpu = wl.pool.k_cache(0).cpu(), wl.pool.v_cache(0).cpu()
+    if wl.mode == "decode":
+        W = wl.group.num_workers
+        n = min(W, sample)
+        group = WorkerGroup(wl.group.workers[:n])
+        pending = {id(b): wl.pending[id(b)] for b in group.write_to}
+        slots = wl.new_token_slots.cpu()[:n]
+        plan = oracle_decode_plan(group, pending, slots, P)
+        q, k, v = wl.q.cpu()[:n], wl.k.cpu()[:n], wl.v.cpu()[:n]
+        pos = wl.batch.positions.cpu()[:n]
+        logical = sum(plan.seq_lens) + len(plan.aux_slots)
+
+        def run():
+            k_rot = rope.rotate(k.view(n, Hkv, D), pos)
+            O.store_kv(k_cpu.view(-1, Hkv * D), v_cpu.view(-1, Hkv * D), slots, k_rot.reshape(n, -1), v)
+            return O.forward_decode(plan, q.view(n, Hq, D), k_cpu, v_cpu, rope)[0]
+
+        # compulsory bytes of the sample: distinct blocks once
+        distinct = {}
+        for view in group.cache_structure:
+            for b in view:
+                distinct[id(b)] = b.num_tokens + (1 if id(b) in pending else 0)
+        sample_bytes = 2 * Hkv * D * q.element_size() * sum(distinct.values())
+        what = f"first {n} of {W} requests ({logical} logical KV tokens)"
+    else:
+        n = min(len(wl.specs), sample)
+        specs = wl.specs[:n]
+        plan = oracle_prefill_plan(specs, P)
+        rows = plan.num_rows
+        q, k, v = wl.q.cpu()[:rows], wl.k.cpu()[:rows], wl.v.cpu()[:rows]
+        pos = wl.batch.positions.cpu()[:rows]
+        out_loc = wl.batch.out_loc.cpu()[:rows]
+
+        def run():
+            k_rot = rope.rotate(k.view(rows, Hkv, D), pos)
+            O.store_kv(k_cpu.view(-1, Hkv * D), v_cpu.view(-1, Hkv * D), out_loc, k_rot.reshape(rows, -1), v)
+            return O.forward_prefill_batch(plan, q.view(rows, Hq, D), k_cpu, v_cpu, rope)[0]
+
+        sample_bytes = None
+        what = f"first {n} of {len(wl.specs)} requests"
+    run()
+    reps = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        run()
+        reps.append(time.perf_counter() - t0)
+    t = sorted(reps)[1]
+    return t, sample_bytes, cores, what, n
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: view attention runs on a single MI355X here (no collectives, "
+              "no sharding); run with --gpus 1", file=sys.stderr)
+        return 2
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    wl = build_workload(args.workload, dev, args.layers, args.kernel)
+    layers = args.layers
+
+    # whole step (store + attention + merge), wall clock around K steps
+    for i in range(args.warmup):
+        wl.forward(i % layers)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        wl.forward(i % layers)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    kern_avg_ms, kern_med_ms = time_attention_kernel(wl, args.steps, args.warmup, layers)
+    counts = wl.meta.launch.counts
+    decode = wl.mode == "decode"
+    if decode:
+        metric, unit = "view_attention_decode_hbm_gbps", "GB/s"
+        value = wl.alg_bytes / (ms_per_step * 1e-3) / 1e9
+        achieved = wl.alg_bytes / (kern_avg_ms * 1e-3) / 1e9
+        roof = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None)
+    else:
+        metric, unit = "view_attention_prefill_mfma_tflops", "TFLOP/s"
+        value = wl.alg_flops / (ms_per_step * 1e-3) / 1e12
+        achieved = wl.alg_flops / (kern_avg_ms * 1e-3) / 1e12
+        roof = dict(bound="mfma", achieved=round(achieved, 2), peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
+                    frac=round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), traffic=None)
+    roof.update(kernel="attention launch (all work items) + merge", kernel_ms_avg=round(kern_avg_ms, 4),
+                kernel_ms_median=round(kern_med_ms, 4))
+
+    line = {
+        "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": str(wl.op.dtype).replace("torch.", "").replace("bfloat16", "bf16")
+        .replace("float32", "f32").replace("float16", "f16"),
+        "data": "synthetic",
+        "config": {"workload": wl.name, "rows": wl.info.get("rows"), "q_heads": wl.op.num_qo_heads,
+                   "kv_heads": wl.op.num_kv_heads, "head_dim": wl.op.head_dim, "page_size": wl.op.page_size,
+                   "kv_pool_copies": layers, "alg_bytes": wl.alg_bytes, "logical_bytes": wl.logical_bytes,
+                   "alg_flops": wl.alg_flops,
+                   "kernel_family": {1: "generic", 2: "mfma"}.get(counts.kernel), "work_items": counts.n_items,
+                   "kv_chunk": counts.kv_chunk, "q_tile": counts.q_tile, "partials": counts.n_partials},
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        sample = args.cpu_sample or (8 if decode else 1)
+        t_cpu, sample_bytes, cores, what, n = cpu_baseline(wl, sample)
+        if decode:
+            cpu_value, cpu_unit = sample_bytes / t_cpu / 1e9, "GB/s"
+        else:
+            per_req = wl.alg_flops / len(wl.specs)
+            cpu_value, cpu_unit = per_req * n / t_cpu / 1e12, "TFLOP/s"
+        line["cpu_baseline"] = {"value": round(cpu_value, 4), "unit": cpu_unit, "cores": cores, "kind": "port",
+                                "sample": what + f", {t_cpu:.2f} s per pass, torch CPU oracle, median of 3"}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

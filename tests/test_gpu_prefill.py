@@ -1,0 +1,91 @@
+"""GPU parity of view-conditioned prefill: product op vs the CPU oracle.
+Scenarios follow tests/core/test_shared_prefill_attention_graph.py:14-135 of
+the reference (ragged requests, 0..3 context blocks, non-empty write blocks,
+3-D mRoPE positions on some requests) plus scaled configuration 3."""
+
+import pytest
+import torch
+
+from async_llm_amd import workloads
+from async_llm_amd.shared_cache import CacheBlock, PrefillSpec
+from oracle import view_attention_oracle as O
+from tests.util import assert_close, make_op_and_pool, oracle_prefill_plan, oracle_rope, run_prefill_parity
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda")
+KERNELS = ["generic", "auto"]
+
+
+def common_blocks(page, mrope):
+    blocks = []
+    for start, length in zip((0, 2, 5), (17, 35, 9)):
+        b = CacheBlock(DEV, page)
+        b.grow_pages(torch.arange(start, start + -(-length // page)) * page, length)
+        if mrope:
+            b.mrope_span_override = length // 2 + 1
+        blocks.append(b)
+    return blocks
+
+
+def make_specs(common, lengths, turn, page, mrope, full_context=False, depth=3):
+    specs = []
+    for worker, length in enumerate(lengths):
+        prefix = (worker * 7 + turn) % 14
+        pages = torch.arange(10 + worker * 12, 10 + worker * 12 + -(-(prefix + length) // page), dtype=torch.int32) * page
+        rel = None
+        if mrope and (worker + turn) % 2:
+            p = torch.arange(length)
+            rel = torch.stack([p // 8, p // 4, p % 4])
+        own_span = prefix // 2 if mrope else prefix
+        context = [common[(turn + j) % 3] for j in range(depth if full_context else (worker + turn) % 4)]
+        specs.append(PrefillSpec(context, pages, length, prefix, own_span, rel))
+    return specs
+
+
+@pytest.mark.parametrize("kernel", KERNELS)
+@pytest.mark.parametrize("mrope", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_ragged_prefill_batches(kernel, mrope, dtype):
+    page, heads = 16, (4, 2, 64)
+    op, cpu_pool, dev_pool, gen = make_op_and_pool(
+        DEV, dtype, heads, page, 64, 1e4, rotary_dim=32 if mrope else 64,
+        mrope_section=(8, 4, 4) if mrope else None, seed=734, scale=1.0, kernel=kernel, max_pos=2048)
+    common = common_blocks(page, mrope)
+    for turn, lengths in ((0, [1]), (2, [63, 65, 3]), (3, [138, 91, 1]), (4, [64] * 4), (5, [9, 7])):
+        specs = make_specs(common, lengths, turn, page, mrope, full_context=(turn == 4))
+        run_prefill_parity(op, cpu_pool, dev_pool, specs, 1e4, gen, scale=1.0)
+
+
+@pytest.mark.parametrize("kernel", KERNELS)
+def test_plain_prefill_without_context(kernel):
+    page = 16
+    op, cpu_pool, dev_pool, gen = make_op_and_pool(DEV, torch.bfloat16, (8, 2, 128), page, 64, 1e6, seed=5,
+                                                   kernel=kernel)
+    specs = [PrefillSpec([], torch.arange(0, 9, dtype=torch.int32) * page, 130),
+             PrefillSpec([], torch.arange(20, 22, dtype=torch.int32) * page, 5, 20)]
+    *_, meta = run_prefill_parity(op, cpu_pool, dev_pool, specs, 1e6, gen)
+    assert meta.n_ctx_rows == 0 and meta.max_segments == 1
+
+
+@pytest.mark.parametrize("kernel", KERNELS)
+def test_scaled_view_prefill_configuration(kernel):
+    """Configuration 3 at reduced size: every request extends its own block and
+    reads the prompt plus the other requests' blocks at their pre-write length."""
+    wl = workloads.view_prefill(DEV, requests=3, new_tokens=96, own_prefix=40, prompt_len=300, kernel=kernel)
+    op = wl.op
+    Hq, Hkv, D, P = op.num_qo_heads, op.num_kv_heads, op.head_dim, op.page_size
+    k_cpu, v_cpu = wl.pool.k_cache(0).cpu(), wl.pool.v_cache(0).cpu()
+    out, lse = op.forward_with_lse(wl.q, wl.k, wl.v, 0, wl.batch)
+    oplan = oracle_prefill_plan(wl.specs, P)
+    assert torch.equal(wl.meta.sub_loc.cpu(), oplan.sub_loc)
+    rope = oracle_rope(op, wl.theta)
+    N = wl.q.shape[0]
+    k_rot = rope.rotate(wl.k.cpu().view(N, Hkv, D), wl.batch.positions.cpu())
+    O.store_kv(k_cpu.view(-1, Hkv * D), v_cpu.view(-1, Hkv * D), wl.batch.out_loc.cpu(), k_rot.reshape(N, -1), wl.v.cpu())
+    assert torch.equal(wl.pool.k_cache(0).cpu(), k_cpu)
+    eo, el = O.forward_prefill_batch(oplan, wl.q.cpu().view(N, Hq, D), k_cpu, v_cpu, rope)
+    assert_close(out, eo, op.dtype, "out")
+    assert_close(lse, el, op.dtype, "lse")
+    pairs = 3 * (96 * (300 + 2 * 40) + 96 * 40 + 96 * 97 // 2)
+    assert wl.alg_flops == 4 * D * Hq * pairs
+    assert wl.meta.last_indices.tolist() == [95, 191, 287]
