@@ -1,18 +1,345 @@
-// Matrix-core (MFMA) attention kernels for 16-bit element types.
+// Matrix-core (MFMA) view attention for 16-bit element types on gfx950.
+//
+// One workgroup of four waves per (work item, kv head).  The item's query tile
+// is at most 16 MFMA rows: row j = (tile row j / G, head j % G) with G = q heads
+// per kv head, so a decode tile batches 16/G requests that read the same KV run.
+// Each wave streams every fourth 32-token tile of the chain:
+//
+//   S^T[token, row]  = K[token, :] . Q^T[:, row]        v_mfma_f32_16x16x32, K as the A operand
+//   online softmax per row (row = lane % 16, so all of a lane's scores share a row)
+//   O^T[dim, row]   += V^T[dim, token] . P^T[token, row] V as the A operand, P as the B operand
+//
+// K fragments are loaded straight into the A-operand layout (16 bytes per lane).
+// The S^T accumulator layout (lane holds tokens 4*(lane/16)+r of each 16-token
+// half) is exactly the B-operand layout of P once the contraction index of the
+// second product is permuted accordingly, so P never moves between lanes.  V is
+// loaded so that the 16 lanes of a group read one contiguous run of a token row;
+// the 8-token x (D/16)-dim block each lane holds is transposed in registers with
+// v_perm_b32 into A operands.  The query tile is rotated for the current link
+// (sub-request) by all 256 threads into LDS and read back as B operands.
+// Wave states are merged through LDS; the result goes to `out` or to a partial
+// slot for the merge kernel.
 #include <hip/hip_runtime.h>
 
 #include "va_internal.h"
 #include "va_launch.h"
 
+typedef __bf16 va_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 va_f16x8 __attribute__((ext_vector_type(8)));
+typedef float va_f32x4 __attribute__((ext_vector_type(4)));
+
 bool va_mfma_supported(int dtype, int head_dim, int gqa) {
-  (void)dtype; (void)head_dim; (void)gqa;
-  return false;
+  if (dtype != VA_BF16 && dtype != VA_F16) return false;
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256) return false;
+  return gqa == 1 || gqa == 2 || gqa == 4 || gqa == 8 || gqa == 16;
 }
-int va_mfma_max_q_tile(int gqa) { return 16 / (gqa > 16 ? 16 : gqa); }
-int va_mfma_default_q_tile(int gqa, bool has_chain) { (void)has_chain; return va_mfma_max_q_tile(gqa); }
+int va_mfma_max_q_tile(int gqa) { return 16 / gqa; }
+int va_mfma_default_q_tile(int gqa, bool has_chain) {
+  (void)has_chain;
+  return 16 / gqa;
+}
 
 namespace va {
-int launch_mfma(const AttnArgs&, int, int, int, hipStream_t) {
-  return va_fail(VA_ERR_ARG, "matrix-core path not available for this configuration");
+
+template <typename E>
+struct Mma;
+template <>
+struct Mma<BF16> {
+  static __device__ __forceinline__ va_f32x4 run(const uint4& a, const uint4& b, va_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(va_bf16x8, a), __builtin_bit_cast(va_bf16x8, b),
+                                                   c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    const __bf16 l = (__bf16)lo, h = (__bf16)hi;
+    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+  }
+};
+template <>
+struct Mma<F16> {
+  static __device__ __forceinline__ va_f32x4 run(const uint4& a, const uint4& b, va_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(va_f16x8, a), __builtin_bit_cast(va_f16x8, b), c,
+                                                  0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    const _Float16 l = (_Float16)lo, h = (_Float16)hi;
+    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+  }
+};
+
+constexpr int kMfmaThreads = 256;
+constexpr int kMfmaWaves = 4;
+constexpr int kTileTokens = 32;
+
+template <typename E, int kD>
+__global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
+  using S = typename E::storage;
+  constexpr int kSteps = kD / 32;   // contraction steps of Q.K^T
+  constexpr int kDimTiles = kD / 16;  // 16-dim tiles of the output
+  constexpr int kChunks = kD / 8;   // 16-byte pieces of a head row
+  constexpr int kVDw = kD / 32;     // dwords of a V token a lane holds (D/16 dims)
+
+  __shared__ uint4 q_s[16][kChunks + 1];
+  __shared__ float o_s[2][16][kD + 4];
+  __shared__ float ml_s[2][16][2];
+
+  const int32_t* item = a.items + (long long)blockIdx.x * VA_ITEM_WORDS;
+  const int hk = blockIdx.y;
+  const int G = a.num_q_heads / a.num_kv_heads;
+  const int n_q = item[VA_I_N_Q];
+  const int part_base = item[VA_I_PART_BASE];
+  const int tid = threadIdx.x;
+  const int wave = tid / kWave;
+  const int lane = tid % kWave;
+  const int j = lane % 16;   // MFMA row of this lane: tile row j / G, head j % G
+  const int kg = lane / 16;  // contraction group
+  const int row_iq = j / G;
+  const S* kp = (const S*)a.k_pool;
+  const S* vp = (const S*)a.v_pool;
+
+  float m_run = kNegBig, l_run = 0.f;
+  va_f32x4 o[kDimTiles];
+#pragma unroll
+  for (int t = 0; t < kDimTiles; ++t) o[t] = va_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int li = 0; li < item[VA_I_N_LINKS]; ++li) {
+    const int32_t* link = a.links + (long long)(item[VA_I_LINK_BEGIN] + li) * VA_LINK_WORDS;
+    const int lflags = link[VA_L_FLAGS];
+    const int qref = link[VA_L_QREF];
+    const int kv_begin = link[VA_L_KV_BEGIN];
+    const int tok_end = link[VA_L_TOK_END];
+    const int causal_base = link[VA_L_CAUSAL_BASE];
+    const bool slots = lflags & VA_LINK_SLOTS;
+
+    // ---- rotate the query tile for this link into LDS ----
+    __syncthreads();
+    for (int idx = tid; idx < 16 * kChunks; idx += kMfmaThreads) {
+      const int jr = idx / kChunks, c = idx - jr * kChunks;
+      const int iq = jr / G, g = jr - iq * G;
+      uint4 packed = make_uint4(0, 0, 0, 0);
+      if (iq < n_q) {
+        const int subrow = (lflags & VA_LINK_INDIRECT) ? a.qrefs[qref + iq] : qref + iq;
+        const long long src_row = a.sub_worker[subrow];
+        const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
+        const int d0 = c * 8;
+        if (d0 < a.rope.rotary_dim) {
+          const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
+          const bool first = d0 < a.rope.half;
+          const int i0 = first ? d0 : d0 - a.rope.half;
+          const uint4 ra = *(const uint4*)(qh + i0);
+          const uint4 rb = *(const uint4*)(qh + i0 + a.rope.half);
+          const S* xa = (const S*)&ra;
+          const S* xb = (const S*)&rb;
+          S res[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            float cs, sn, y1, y2;
+            rope_cos_sin(a.rope, p, i0 + e, cs, sn);
+            rope_pair<E>(a.rope, cs, sn, E::load(xa[e]), E::load(xb[e]), y1, y2);
+            res[e] = E::store(first ? y1 : y2);
+          }
+          packed = *(const uint4*)res;
+        } else {
+          packed = *(const uint4*)(qh + d0);
+        }
+      }
+      q_s[jr][c] = packed;
+    }
+    __syncthreads();
+    uint4 qf[kSteps];
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) qf[s] = q_s[j][4 * s + kg];
+
+    // visible range of this link for the tile and for this lane's row
+    const int t_stop = min(tok_end, causal_base + n_q);
+    const int t_row = min(tok_end, causal_base + row_iq + 1);
+    const int t_last = t_stop - 1;
+
+    for (int t0 = link[VA_L_TOK_BEGIN] + wave * kTileTokens; t0 < t_stop; t0 += kMfmaWaves * kTileTokens) {
+      // ---- K fragments: lane (j, kg) holds dims [32s + 8kg, +8) of tokens t0 + j and t0 + 16 + j ----
+      uint4 kf[2][kSteps];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int t = min(t0 + 16 * u + j, t_last);
+        const long long slot = kv_slot(a.kv_indices, kv_begin, t, a.page_size, slots);
+        const S* kr = kp + slot * a.pool_row_stride + (long long)hk * kD + 8 * kg;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) kf[u][s] = *(const uint4*)(kr + 32 * s);
+      }
+      // ---- V block: lane (j, kg) holds dims [j*D/16, +D/16) of the 8 tokens it scored ----
+      uint32_t vraw[8][kVDw];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int t = min(t0 + 16 * (e / 4) + 4 * kg + (e % 4), t_last);
+        const long long slot = kv_slot(a.kv_indices, kv_begin, t, a.page_size, slots);
+        const S* vr = vp + slot * a.pool_row_stride + (long long)hk * kD + j * (kD / 16);
+        if constexpr (kVDw == 8) {
+          const uint4 x = *(const uint4*)vr, y = *(const uint4*)(vr + 8);
+          vraw[e][0] = x.x; vraw[e][1] = x.y; vraw[e][2] = x.z; vraw[e][3] = x.w;
+          vraw[e][4] = y.x; vraw[e][5] = y.y; vraw[e][6] = y.z; vraw[e][7] = y.w;
+        } else if constexpr (kVDw == 4) {
+          const uint4 x = *(const uint4*)vr;
+          vraw[e][0] = x.x; vraw[e][1] = x.y; vraw[e][2] = x.z; vraw[e][3] = x.w;
+        } else {
+          const uint2 x = *(const uint2*)vr;
+          vraw[e][0] = x.x; vraw[e][1] = x.y;
+        }
+      }
+
+      // ---- scores ----
+      va_f32x4 sc[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        sc[u] = va_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) sc[u] = Mma<E>::run(kf[u][s], qf[s], sc[u]);
+      }
+      float tile_max = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int t = t0 + 16 * u + 4 * kg + r;
+          const float v = t < t_row ? sc[u][r] * a.scale_log2 : -INFINITY;
+          sc[u][r] = v;
+          tile_max = fmaxf(tile_max, v);
+        }
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+      const float m_new = fmaxf(m_run, tile_max);
+      const float alpha = exp2f(m_run - m_new);
+      m_run = m_new;
+      float psum = 0.f;
+      float pr[8];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float p = exp2f(sc[u][r] - m_new);
+          pr[4 * u + r] = p;
+          psum += p;
+        }
+      l_run = l_run * alpha + psum;
+      if (__any(alpha != 1.f)) {
+#pragma unroll
+        for (int t = 0; t < kDimTiles; ++t) o[t] *= alpha;
+      }
+      uint4 pf;
+      pf.x = Mma<E>::pack(pr[0], pr[1]);
+      pf.y = Mma<E>::pack(pr[2], pr[3]);
+      pf.z = Mma<E>::pack(pr[4], pr[5]);
+      pf.w = Mma<E>::pack(pr[6], pr[7]);
+
+      // ---- O^T += V^T . P^T, one 16-dim tile at a time; tile T takes element T of the lane's run ----
+#pragma unroll
+      for (int t = 0; t < kDimTiles; ++t) {
+        const int w = t / 2;
+        const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
+        uint4 vf;
+        vf.x = __builtin_amdgcn_perm(vraw[1][w], vraw[0][w], sel);
+        vf.y = __builtin_amdgcn_perm(vraw[3][w], vraw[2][w], sel);
+        vf.z = __builtin_amdgcn_perm(vraw[5][w], vraw[4][w], sel);
+        vf.w = __builtin_amdgcn_perm(vraw[7][w], vraw[6][w], sel);
+        o[t] = Mma<E>::run(vf, pf, o[t]);
+      }
+    }
+  }
+
+  // row sums live spread over the four contraction groups
+  l_run += __shfl_xor(l_run, 16, kWave);
+  l_run += __shfl_xor(l_run, 32, kWave);
+
+  // ---- merge the four waves: (2,3) -> LDS, (0,1) fold them in, 1 -> LDS, 0 folds and emits ----
+  auto spill = [&](int buf) {
+#pragma unroll
+    for (int t = 0; t < kDimTiles; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o_s[buf][j][(4 * kg + r) * (kD / 16) + t] = o[t][r];
+    if (kg == 0) {
+      ml_s[buf][j][0] = m_run;
+      ml_s[buf][j][1] = l_run;
+    }
+  };
+  auto fold = [&](int buf) {
+    const float m_o = ml_s[buf][j][0], l_o = ml_s[buf][j][1];
+    const float m_new = fmaxf(m_run, m_o);
+    const float sa = exp2f(m_run - m_new), sb = exp2f(m_o - m_new);
+    l_run = l_run * sa + l_o * sb;
+    m_run = m_new;
+#pragma unroll
+    for (int t = 0; t < kDimTiles; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[t][r] = o[t][r] * sa + o_s[buf][j][(4 * kg + r) * (kD / 16) + t] * sb;
+  };
+  __syncthreads();
+  if (wave >= 2) spill(wave - 2);
+  __syncthreads();
+  if (wave < 2) fold(wave);
+  __syncthreads();
+  if (wave == 1) spill(0);
+  __syncthreads();
+  if (wave == 0) {
+    fold(0);
+    spill(1);
+  }
+  __syncthreads();
+
+  // ---- emit: all threads, coalesced over the head dimension ----
+  for (int idx = tid; idx < 16 * kD; idx += kMfmaThreads) {
+    const int jr = idx / kD, d = idx - jr * kD;
+    const int iq = jr / G, g = jr - iq * G;
+    if (iq >= n_q) continue;
+    const int hq = hk * G + g;
+    const float mm = ml_s[1][jr][0], ll = ml_s[1][jr][1];
+    const float av = o_s[1][jr][d];
+    if (part_base < 0) {
+      const int32_t* link = a.links + (long long)item[VA_I_LINK_BEGIN] * VA_LINK_WORDS;
+      const int subrow = (link[VA_L_FLAGS] & VA_LINK_INDIRECT) ? a.qrefs[link[VA_L_QREF] + iq] : link[VA_L_QREF] + iq;
+      const long long out_row = a.sub_worker[subrow];
+      ((S*)a.out)[(out_row * a.num_q_heads + hq) * (long long)kD + d] = E::store(ll > 0.f ? av / ll : 0.f);
+      if (d == 0 && a.lse) {
+        const float lse2 = ll > 0.f ? mm + log2f(ll) : -INFINITY;
+        a.lse[out_row * a.num_q_heads + hq] = a.lse_base2 ? lse2 : lse2 * kLn2;
+      }
+    } else {
+      const long long slot = (long long)(part_base + iq) * a.num_q_heads + hq;
+      a.part_acc[slot * kD + d] = av;
+      if (d == 0) {
+        a.part_ml[slot * 2 + 0] = mm;
+        a.part_ml[slot * 2 + 1] = ll;
+      }
+    }
+  }
 }
+
+template <typename E>
+static int launch_mfma_typed(const AttnArgs& a, int n_items, hipStream_t stream) {
+  const dim3 grid((unsigned)n_items, (unsigned)a.num_kv_heads), block(kMfmaThreads);
+  switch (a.head_dim) {
+    case 64:
+      hipLaunchKernelGGL((attn_mfma_kernel<E, 64>), grid, block, 0, stream, a);
+      break;
+    case 128:
+      hipLaunchKernelGGL((attn_mfma_kernel<E, 128>), grid, block, 0, stream, a);
+      break;
+    case 256:
+      hipLaunchKernelGGL((attn_mfma_kernel<E, 256>), grid, block, 0, stream, a);
+      break;
+    default:
+      return va_fail(VA_ERR_ARG, "matrix-core path supports head_dim 64, 128, 256");
+  }
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? VA_OK : va_fail(VA_ERR_HIP, "attention launch: %s", hipGetErrorString(e));
+}
+
+int launch_mfma(const AttnArgs& a, int dtype, int n_items, int q_tile, hipStream_t stream) {
+  const int g = a.num_q_heads / a.num_kv_heads;
+  if (!va_mfma_supported(dtype, a.head_dim, g))
+    return va_fail(VA_ERR_ARG, "matrix-core path does not support this dtype/head_dim/group size");
+  if (q_tile * g > 16) return va_fail(VA_ERR_ARG, "plan tile of %d rows x %d heads exceeds 16 MFMA rows", q_tile, g);
+  if (a.rope.rotary_dim % 16) return va_fail(VA_ERR_ARG, "matrix-core path needs rotary_dim to be a multiple of 16");
+  if (a.q_row_stride % 8 || a.pool_row_stride % 8)
+    return va_fail(VA_ERR_ARG, "matrix-core path needs 16-byte aligned rows");
+  return dtype == VA_BF16 ? launch_mfma_typed<BF16>(a, n_items, stream) : launch_mfma_typed<F16>(a, n_items, stream);
+}
+
 }  // namespace va

@@ -164,6 +164,8 @@ class SharedCacheAttention:
         kernel = kernel or os.environ.get("VIEWATTN_KERNEL", "auto")
         if kernel not in _KERNELS:
             raise ValueError(f"kernel must be one of {sorted(_KERNELS)}, got {kernel!r}")
+        if kernel == "auto" and self.rotary_dim % 16:
+            kernel = "generic"  # the matrix-core kernel rotates queries in 8-element pieces
         self.kernel = kernel
         self.plan_params = native.VaPlanParams(_KERNELS[kernel], 0, 0, 0)
         self._shape = native.make_shape(num_qo_heads, num_kv_heads, head_dim, page_size, dtype)
