@@ -28,23 +28,24 @@ HIPCC_FLAGS = [
 ]
 
 
-def build(verbose: bool = True) -> str:
+def build(verbose: bool = True, out: str = LIB_PATH, extra_flags=()) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *HIPCC_FLAGS, "-DVA_BUILDING=1"]
+    cmd = [hipcc, *HIPCC_FLAGS, "-DVA_BUILDING=1", *extra_flags]
     for src in SOURCES:
         path = os.path.join(CSRC, src)
         if src.endswith(".cpp"):
             cmd += ["-x", "hip", path]
         else:
             cmd.append(path)
-    cmd += ["-o", LIB_PATH]
+    cmd += ["-o", out]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True, cwd=CSRC)
-    return LIB_PATH
+    return out
 
 
 if __name__ == "__main__":
-    build()
-    print(LIB_PATH)
+    # usage: build.py [output.so [extra hipcc flags...]]
+    target = os.path.abspath(sys.argv[1]) if len(sys.argv) > 1 else LIB_PATH
+    print(build(out=target, extra_flags=sys.argv[2:]))
     sys.exit(0)

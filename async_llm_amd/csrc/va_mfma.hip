@@ -17,6 +17,15 @@
 // the 8-token x (D/16)-dim block each lane holds is transposed in registers with
 // v_perm_b32 into A operands.  The query tile is rotated for the current link
 // (sub-request) by all 256 threads into LDS and read back as B operands.
+//
+// Memory pipeline: the K registers are free as soon as the scores are computed
+// and the V registers as soon as the output is updated, so the loads of the next
+// tile's K are issued right after Q.K^T and those of its V right after P.V; a
+// wave always has 16-32 KB of loads in flight while it computes, at no register
+// cost.  Page-table entries are wave-uniform when the page size is a multiple of
+// 16 (a 16-token half tile never straddles a page) and are fetched with scalar
+// loads one tile ahead.
+//
 // Wave states are merged through LDS; the result goes to `out` or to a partial
 // slot for the merge kernel.
 #include <hip/hip_runtime.h>
@@ -70,13 +79,18 @@ constexpr int kMfmaThreads = 256;
 constexpr int kMfmaWaves = 4;
 constexpr int kTileTokens = 32;
 
+#ifndef VA_MFMA_MIN_BLOCKS
+#define VA_MFMA_MIN_BLOCKS 2  // workgroups per CU the register allocation must allow
+#endif
+
 template <typename E, int kD>
-__global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
+__global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_kernel(AttnArgs a) {
   using S = typename E::storage;
-  constexpr int kSteps = kD / 32;   // contraction steps of Q.K^T
+  constexpr int kSteps = kD / 32;     // contraction steps of Q.K^T
   constexpr int kDimTiles = kD / 16;  // 16-dim tiles of the output
-  constexpr int kChunks = kD / 8;   // 16-byte pieces of a head row
-  constexpr int kVDw = kD / 32;     // dwords of a V token a lane holds (D/16 dims)
+  constexpr int kChunks = kD / 8;     // 16-byte pieces of a head row
+  constexpr int kVDw = kD / 32;       // dwords of a V token a lane holds (D/16 dims)
+  constexpr int kStride = kMfmaWaves * kTileTokens;
 
   __shared__ uint4 q_s[16][kChunks + 1];
   __shared__ float o_s[2][16][kD + 4];
@@ -88,13 +102,14 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const int n_q = item[VA_I_N_Q];
   const int part_base = item[VA_I_PART_BASE];
   const int tid = threadIdx.x;
-  const int wave = tid / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int lane = tid % kWave;
   const int j = lane % 16;   // MFMA row of this lane: tile row j / G, head j % G
   const int kg = lane / 16;  // contraction group
   const int row_iq = j / G;
-  const S* kp = (const S*)a.k_pool;
-  const S* vp = (const S*)a.v_pool;
+  const S* kp = (const S*)a.k_pool + (long long)hk * kD + 8 * kg;         // + row*stride + 32*s
+  const S* vp = (const S*)a.v_pool + (long long)hk * kD + j * (kD / 16);  // + row*stride
+  const int P = a.page_size;
 
   float m_run = kNegBig, l_run = 0.f;
   va_f32x4 o[kDimTiles];
@@ -109,6 +124,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     const int tok_end = link[VA_L_TOK_END];
     const int causal_base = link[VA_L_CAUSAL_BASE];
     const bool slots = lflags & VA_LINK_SLOTS;
+    const bool uniform_pages = !slots && (P % 16 == 0);
 
     // ---- rotate the query tile for this link into LDS ----
     __syncthreads();
@@ -145,33 +161,42 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       q_s[jr][c] = packed;
     }
     __syncthreads();
-    uint4 qf[kSteps];
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s) qf[s] = q_s[j][4 * s + kg];
 
     // visible range of this link for the tile and for this lane's row
     const int t_stop = min(tok_end, causal_base + n_q);
     const int t_row = min(tok_end, causal_base + row_iq + 1);
     const int t_last = t_stop - 1;
 
-    for (int t0 = link[VA_L_TOK_BEGIN] + wave * kTileTokens; t0 < t_stop; t0 += kMfmaWaves * kTileTokens) {
-      // ---- K fragments: lane (j, kg) holds dims [32s + 8kg, +8) of tokens t0 + j and t0 + 16 + j ----
-      uint4 kf[2][kSteps];
+    // Pool rows of the two 16-token halves of the tile starting at t0 (uniform pages):
+    // row of token min(t0 + 16u, t_last) rounded down to its 16-token group.  Every
+    // clamped token of the half lies in that group, so lanes only add their offset.
+    auto half_rows = [&](int t0, long long (&rows)[2]) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int t = min(t0 + 16 * u, t_last);
+        const int page = __builtin_amdgcn_readfirstlane(a.kv_indices[kv_begin + t / P]);
+        rows[u] = (long long)page * P + ((t % P) & ~15);
+      }
+    };
+    // K fragments: lane (j, kg) holds dims [32s + 8kg, +8) of tokens t0 + j and t0 + 16 + j.
+    auto load_k = [&](int t0, const long long (&rows)[2], uint4 (&kf)[2][kSteps]) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         const int t = min(t0 + 16 * u + j, t_last);
-        const long long slot = kv_slot(a.kv_indices, kv_begin, t, a.page_size, slots);
-        const S* kr = kp + slot * a.pool_row_stride + (long long)hk * kD + 8 * kg;
+        const long long row = uniform_pages ? rows[u] + (t & 15) : kv_slot(a.kv_indices, kv_begin, t, P, slots);
+        const S* kr = kp + row * a.pool_row_stride;
 #pragma unroll
         for (int s = 0; s < kSteps; ++s) kf[u][s] = *(const uint4*)(kr + 32 * s);
       }
-      // ---- V block: lane (j, kg) holds dims [j*D/16, +D/16) of the 8 tokens it scored ----
-      uint32_t vraw[8][kVDw];
+    };
+    // V block: lane (j, kg) holds dims [j*D/16, +D/16) of the 8 tokens it scores:
+    // t0 + 16*(e/4) + 4*kg + e%4, e = 0..7.
+    auto load_v = [&](int t0, const long long (&rows)[2], uint32_t (&vraw)[8][kVDw]) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int t = min(t0 + 16 * (e / 4) + 4 * kg + (e % 4), t_last);
-        const long long slot = kv_slot(a.kv_indices, kv_begin, t, a.page_size, slots);
-        const S* vr = vp + slot * a.pool_row_stride + (long long)hk * kD + j * (kD / 16);
+        const long long row = uniform_pages ? rows[e / 4] + (t & 15) : kv_slot(a.kv_indices, kv_begin, t, P, slots);
+        const S* vr = vp + row * a.pool_row_stride;
         if constexpr (kVDw == 8) {
           const uint4 x = *(const uint4*)vr, y = *(const uint4*)(vr + 8);
           vraw[e][0] = x.x; vraw[e][1] = x.y; vraw[e][2] = x.z; vraw[e][3] = x.w;
@@ -184,62 +209,83 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
           vraw[e][0] = x.x; vraw[e][1] = x.y;
         }
       }
+    };
 
-      // ---- scores ----
-      va_f32x4 sc[2];
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        sc[u] = va_f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < kSteps; ++s) sc[u] = Mma<E>::run(kf[u][s], qf[s], sc[u]);
-      }
-      float tile_max = -INFINITY;
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int t = t0 + 16 * u + 4 * kg + r;
-          const float v = t < t_row ? sc[u][r] * a.scale_log2 : -INFINITY;
-          sc[u][r] = v;
-          tile_max = fmaxf(tile_max, v);
-        }
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
-      const float m_new = fmaxf(m_run, tile_max);
-      const float alpha = exp2f(m_run - m_new);
-      m_run = m_new;
-      float psum = 0.f;
-      float pr[8];
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float p = exp2f(sc[u][r] - m_new);
-          pr[4 * u + r] = p;
-          psum += p;
-        }
-      l_run = l_run * alpha + psum;
-      if (__any(alpha != 1.f)) {
-#pragma unroll
-        for (int t = 0; t < kDimTiles; ++t) o[t] *= alpha;
-      }
-      uint4 pf;
-      pf.x = Mma<E>::pack(pr[0], pr[1]);
-      pf.y = Mma<E>::pack(pr[2], pr[3]);
-      pf.z = Mma<E>::pack(pr[4], pr[5]);
-      pf.w = Mma<E>::pack(pr[6], pr[7]);
+    int t0 = link[VA_L_TOK_BEGIN] + wave * kTileTokens;
+    if (t0 < t_stop) {
+      uint4 kf[2][kSteps];
+      uint32_t vraw[8][kVDw];
+      long long rows[2] = {0, 0};
+      if (uniform_pages) half_rows(t0, rows);
+      load_k(t0, rows, kf);
+      load_v(t0, rows, vraw);
+      while (true) {
+        const int tn = t0 + kStride;
+        const bool more = tn < t_stop;
+        if (more && uniform_pages) half_rows(tn, rows);
 
-      // ---- O^T += V^T . P^T, one 16-dim tile at a time; tile T takes element T of the lane's run ----
+        // ---- scores: S^T = K . Q^T ----
+        va_f32x4 sc[2];
 #pragma unroll
-      for (int t = 0; t < kDimTiles; ++t) {
-        const int w = t / 2;
-        const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
-        uint4 vf;
-        vf.x = __builtin_amdgcn_perm(vraw[1][w], vraw[0][w], sel);
-        vf.y = __builtin_amdgcn_perm(vraw[3][w], vraw[2][w], sel);
-        vf.z = __builtin_amdgcn_perm(vraw[5][w], vraw[4][w], sel);
-        vf.w = __builtin_amdgcn_perm(vraw[7][w], vraw[6][w], sel);
-        o[t] = Mma<E>::run(vf, pf, o[t]);
+        for (int u = 0; u < 2; ++u) {
+          sc[u] = va_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < kSteps; ++s) sc[u] = Mma<E>::run(kf[u][s], q_s[j][4 * s + kg], sc[u]);
+        }
+        if (more) load_k(tn, rows, kf);  // K registers are free again
+
+        // ---- online softmax (row = lane % 16) ----
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int t = t0 + 16 * u + 4 * kg + r;
+            const float v = t < t_row ? sc[u][r] * a.scale_log2 : -INFINITY;
+            sc[u][r] = v;
+            tile_max = fmaxf(tile_max, v);
+          }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+        const float m_new = fmaxf(m_run, tile_max);
+        const float alpha = exp2f(m_run - m_new);
+        m_run = m_new;
+        float psum = 0.f;
+        float pr[8];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float p = exp2f(sc[u][r] - m_new);
+            pr[4 * u + r] = p;
+            psum += p;
+          }
+        l_run = l_run * alpha + psum;
+        if (__any(alpha != 1.f)) {
+#pragma unroll
+          for (int t = 0; t < kDimTiles; ++t) o[t] *= alpha;
+        }
+        uint4 pf;
+        pf.x = Mma<E>::pack(pr[0], pr[1]);
+        pf.y = Mma<E>::pack(pr[2], pr[3]);
+        pf.z = Mma<E>::pack(pr[4], pr[5]);
+        pf.w = Mma<E>::pack(pr[6], pr[7]);
+
+        // ---- O^T += V^T . P^T, one 16-dim tile at a time; tile T takes element T of the lane's run ----
+#pragma unroll
+        for (int t = 0; t < kDimTiles; ++t) {
+          const int w = t / 2;
+          const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
+          uint4 vf;
+          vf.x = __builtin_amdgcn_perm(vraw[1][w], vraw[0][w], sel);
+          vf.y = __builtin_amdgcn_perm(vraw[3][w], vraw[2][w], sel);
+          vf.z = __builtin_amdgcn_perm(vraw[5][w], vraw[4][w], sel);
+          vf.w = __builtin_amdgcn_perm(vraw[7][w], vraw[6][w], sel);
+          o[t] = Mma<E>::run(vf, pf, o[t]);
+        }
+        if (!more) break;
+        load_v(tn, rows, vraw);  // V registers are free again
+        t0 = tn;
       }
     }
   }
@@ -284,6 +330,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   __syncthreads();
 
   // ---- emit: all threads, coalesced over the head dimension ----
+  const int32_t* link0 = a.links + (long long)item[VA_I_LINK_BEGIN] * VA_LINK_WORDS;
   for (int idx = tid; idx < 16 * kD; idx += kMfmaThreads) {
     const int jr = idx / kD, d = idx - jr * kD;
     const int iq = jr / G, g = jr - iq * G;
@@ -292,8 +339,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     const float mm = ml_s[1][jr][0], ll = ml_s[1][jr][1];
     const float av = o_s[1][jr][d];
     if (part_base < 0) {
-      const int32_t* link = a.links + (long long)item[VA_I_LINK_BEGIN] * VA_LINK_WORDS;
-      const int subrow = (link[VA_L_FLAGS] & VA_LINK_INDIRECT) ? a.qrefs[link[VA_L_QREF] + iq] : link[VA_L_QREF] + iq;
+      const int subrow = (link0[VA_L_FLAGS] & VA_LINK_INDIRECT) ? a.qrefs[link0[VA_L_QREF] + iq] : link0[VA_L_QREF] + iq;
       const long long out_row = a.sub_worker[subrow];
       ((S*)a.out)[(out_row * a.num_q_heads + hq) * (long long)kD + d] = E::store(ll > 0.f ? av / ll : 0.f);
       if (d == 0 && a.lse) {

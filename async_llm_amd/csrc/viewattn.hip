@@ -337,21 +337,40 @@ __global__ __launch_bounds__(64) void merge_kernel(MergeArgs a) {
     if (threadIdx.x == 0 && a.lse) a.lse[row * a.num_q_heads + hq] = -INFINITY;
     return;
   }
+  // One pass with a running (max, sum, accumulator); eight partials per round so
+  // that their loads are all in flight before the first one is folded in.
   const int b = a.row_indptr[row], e = a.row_indptr[row + 1];
-  float mm = kNegBig;
-  for (int i = b; i < e; ++i) mm = fmaxf(mm, a.part_ml[((long long)a.row_ids[i] * a.num_q_heads + hq) * 2]);
-  float ll = 0.f;
-  for (int i = b; i < e; ++i) {
-    const long long slot = (long long)a.row_ids[i] * a.num_q_heads + hq;
-    ll += a.part_ml[slot * 2 + 1] * exp2f(a.part_ml[slot * 2] - mm);
-  }
-  for (int d = threadIdx.x; d < a.head_dim; d += 64) {
-    float av = 0.f;
-    for (int i = b; i < e; ++i) {
+  const int n_d = (a.head_dim + 63) / 64;  // dims per thread: d = threadIdx.x + 64*k (at most 4 for D = 256)
+  float mm = kNegBig, ll = 0.f;
+  float av[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int i0 = b; i0 < e; i0 += 8) {
+    float mp[8], lp[8], ap[8][4];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = min(i0 + u, e - 1);
       const long long slot = (long long)a.row_ids[i] * a.num_q_heads + hq;
-      av += a.part_acc[slot * a.head_dim + d] * exp2f(a.part_ml[slot * 2] - mm);
+      mp[u] = i0 + u < e ? a.part_ml[slot * 2] : kNegBig;
+      lp[u] = i0 + u < e ? a.part_ml[slot * 2 + 1] : 0.f;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int d = threadIdx.x + 64 * k;
+        ap[u][k] = (k < n_d && d < a.head_dim) ? a.part_acc[slot * a.head_dim + d] : 0.f;
+      }
     }
-    o[d] = E::store(ll > 0.f ? av / ll : 0.f);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const float m_new = fmaxf(mm, mp[u]);
+      const float sa = exp2f(mm - m_new), sb = exp2f(mp[u] - m_new);
+      ll = ll * sa + lp[u] * sb;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) av[k] = av[k] * sa + ap[u][k] * sb;
+      mm = m_new;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int d = threadIdx.x + 64 * k;
+    if (d < a.head_dim) o[d] = E::store(ll > 0.f ? av[k] / ll : 0.f);
   }
   if (threadIdx.x == 0 && a.lse) {
     const float lse2 = ll > 0.f ? mm + log2f(ll) : -INFINITY;

@@ -13,7 +13,8 @@ from typing import Optional
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libviewattn.so")
+# VIEWATTN_LIB selects another build of the same library (e.g. an instrumented one)
+LIB_PATH = os.environ.get("VIEWATTN_LIB") or os.path.join(_HERE, "libviewattn.so")
 
 VA_F32, VA_F16, VA_BF16 = 0, 1, 2
 VA_ROPE_TABLE, VA_ROPE_MROPE = 0, 1
