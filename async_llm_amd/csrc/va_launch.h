@@ -43,6 +43,8 @@ struct MergeArgs {
 };
 
 // Matrix-core attention (va_mfma.hip).
-int launch_mfma(const AttnArgs& a, int dtype, int n_items, int q_tile, hipStream_t stream);
+// `n_wide` leading items are wide tiles (va_mfma_wide.hip), the rest narrow ones.
+int launch_mfma(const AttnArgs& a, int dtype, int n_items, int n_wide, int q_tile, hipStream_t stream);
+int launch_mfma_wide(const AttnArgs& a, int dtype, int n_items, hipStream_t stream);
 
 }  // namespace va

@@ -32,10 +32,7 @@
 
 #include "va_internal.h"
 #include "va_launch.h"
-
-typedef __bf16 va_bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 va_f16x8 __attribute__((ext_vector_type(8)));
-typedef float va_f32x4 __attribute__((ext_vector_type(4)));
+#include "va_mfma_common.h"
 
 bool va_mfma_supported(int dtype, int head_dim, int gqa) {
   if (dtype != VA_BF16 && dtype != VA_F16) return false;
@@ -47,33 +44,9 @@ int va_mfma_default_q_tile(int gqa, bool has_chain) {
   (void)has_chain;
   return 16 / gqa;
 }
+int va_mfma_wide_q_tile(int gqa) { return 128 / gqa; }
 
 namespace va {
-
-template <typename E>
-struct Mma;
-template <>
-struct Mma<BF16> {
-  static __device__ __forceinline__ va_f32x4 run(const uint4& a, const uint4& b, va_f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(va_bf16x8, a), __builtin_bit_cast(va_bf16x8, b),
-                                                   c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    const __bf16 l = (__bf16)lo, h = (__bf16)hi;
-    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
-  }
-};
-template <>
-struct Mma<F16> {
-  static __device__ __forceinline__ va_f32x4 run(const uint4& a, const uint4& b, va_f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(va_f16x8, a), __builtin_bit_cast(va_f16x8, b), c,
-                                                  0, 0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    const _Float16 l = (_Float16)lo, h = (_Float16)hi;
-    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
-  }
-};
 
 constexpr int kMfmaThreads = 256;
 constexpr int kMfmaWaves = 4;
@@ -92,7 +65,7 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
   constexpr int kVDw = kD / 32;       // dwords of a V token a lane holds (D/16 dims)
   constexpr int kStride = kMfmaWaves * kTileTokens;
 
-  __shared__ uint4 q_s[16][kChunks + 1];
+  __shared__ va_u32x4 q_s[16][kChunks + 1];
   __shared__ float o_s[2][16][kD + 4];
   __shared__ float ml_s[2][16][2];
 
@@ -131,32 +104,14 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
     for (int idx = tid; idx < 16 * kChunks; idx += kMfmaThreads) {
       const int jr = idx / kChunks, c = idx - jr * kChunks;
       const int iq = jr / G, g = jr - iq * G;
-      uint4 packed = make_uint4(0, 0, 0, 0);
+      va_u32x4 packed = {0, 0, 0, 0};
       if (iq < n_q) {
         const int subrow = (lflags & VA_LINK_INDIRECT) ? a.qrefs[qref + iq] : qref + iq;
         const long long src_row = a.sub_worker[subrow];
         const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
-        const int d0 = c * 8;
-        if (d0 < a.rope.rotary_dim) {
-          const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
-          const bool first = d0 < a.rope.half;
-          const int i0 = first ? d0 : d0 - a.rope.half;
-          const uint4 ra = *(const uint4*)(qh + i0);
-          const uint4 rb = *(const uint4*)(qh + i0 + a.rope.half);
-          const S* xa = (const S*)&ra;
-          const S* xb = (const S*)&rb;
-          S res[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            float cs, sn, y1, y2;
-            rope_cos_sin(a.rope, p, i0 + e, cs, sn);
-            rope_pair<E>(a.rope, cs, sn, E::load(xa[e]), E::load(xb[e]), y1, y2);
-            res[e] = E::store(first ? y1 : y2);
-          }
-          packed = *(const uint4*)res;
-        } else {
-          packed = *(const uint4*)(qh + d0);
-        }
+        const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
+        const uint4 piece = rotated_query_piece<E>(a.rope, qh, c * 8, p);
+        packed = va_u32x4{piece.x, piece.y, piece.z, piece.w};
       }
       q_s[jr][c] = packed;
     }
@@ -179,14 +134,14 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
       }
     };
     // K fragments: lane (j, kg) holds dims [32s + 8kg, +8) of tokens t0 + j and t0 + 16 + j.
-    auto load_k = [&](int t0, const long long (&rows)[2], uint4 (&kf)[2][kSteps]) {
+    auto load_k = [&](int t0, const long long (&rows)[2], va_u32x4 (&kf)[2][kSteps]) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         const int t = min(t0 + 16 * u + j, t_last);
         const long long row = uniform_pages ? rows[u] + (t & 15) : kv_slot(a.kv_indices, kv_begin, t, P, slots);
         const S* kr = kp + row * a.pool_row_stride;
 #pragma unroll
-        for (int s = 0; s < kSteps; ++s) kf[u][s] = *(const uint4*)(kr + 32 * s);
+        for (int s = 0; s < kSteps; ++s) kf[u][s] = *(const va_u32x4*)(kr + 32 * s);
       }
     };
     // V block: lane (j, kg) holds dims [j*D/16, +D/16) of the 8 tokens it scores:
@@ -198,12 +153,12 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
         const long long row = uniform_pages ? rows[e / 4] + (t & 15) : kv_slot(a.kv_indices, kv_begin, t, P, slots);
         const S* vr = vp + row * a.pool_row_stride;
         if constexpr (kVDw == 8) {
-          const uint4 x = *(const uint4*)vr, y = *(const uint4*)(vr + 8);
-          vraw[e][0] = x.x; vraw[e][1] = x.y; vraw[e][2] = x.z; vraw[e][3] = x.w;
-          vraw[e][4] = y.x; vraw[e][5] = y.y; vraw[e][6] = y.z; vraw[e][7] = y.w;
+          const va_u32x4 x = *(const va_u32x4*)vr, y = *(const va_u32x4*)(vr + 8);
+          vraw[e][0] = x[0]; vraw[e][1] = x[1]; vraw[e][2] = x[2]; vraw[e][3] = x[3];
+          vraw[e][4] = y[0]; vraw[e][5] = y[1]; vraw[e][6] = y[2]; vraw[e][7] = y[3];
         } else if constexpr (kVDw == 4) {
-          const uint4 x = *(const uint4*)vr;
-          vraw[e][0] = x.x; vraw[e][1] = x.y; vraw[e][2] = x.z; vraw[e][3] = x.w;
+          const va_u32x4 x = *(const va_u32x4*)vr;
+          vraw[e][0] = x[0]; vraw[e][1] = x[1]; vraw[e][2] = x[2]; vraw[e][3] = x[3];
         } else {
           const uint2 x = *(const uint2*)vr;
           vraw[e][0] = x.x; vraw[e][1] = x.y;
@@ -213,7 +168,7 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
 
     int t0 = link[VA_L_TOK_BEGIN] + wave * kTileTokens;
     if (t0 < t_stop) {
-      uint4 kf[2][kSteps];
+      va_u32x4 kf[2][kSteps];
       uint32_t vraw[8][kVDw];
       long long rows[2] = {0, 0};
       if (uniform_pages) half_rows(t0, rows);
@@ -265,22 +220,18 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
 #pragma unroll
           for (int t = 0; t < kDimTiles; ++t) o[t] *= alpha;
         }
-        uint4 pf;
-        pf.x = Mma<E>::pack(pr[0], pr[1]);
-        pf.y = Mma<E>::pack(pr[2], pr[3]);
-        pf.z = Mma<E>::pack(pr[4], pr[5]);
-        pf.w = Mma<E>::pack(pr[6], pr[7]);
+        const va_u32x4 pf = {Mma<E>::pack(pr[0], pr[1]), Mma<E>::pack(pr[2], pr[3]), Mma<E>::pack(pr[4], pr[5]),
+                             Mma<E>::pack(pr[6], pr[7])};
 
         // ---- O^T += V^T . P^T, one 16-dim tile at a time; tile T takes element T of the lane's run ----
 #pragma unroll
         for (int t = 0; t < kDimTiles; ++t) {
           const int w = t / 2;
           const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
-          uint4 vf;
-          vf.x = __builtin_amdgcn_perm(vraw[1][w], vraw[0][w], sel);
-          vf.y = __builtin_amdgcn_perm(vraw[3][w], vraw[2][w], sel);
-          vf.z = __builtin_amdgcn_perm(vraw[5][w], vraw[4][w], sel);
-          vf.w = __builtin_amdgcn_perm(vraw[7][w], vraw[6][w], sel);
+          const va_u32x4 vf = {__builtin_amdgcn_perm(vraw[1][w], vraw[0][w], sel),
+                               __builtin_amdgcn_perm(vraw[3][w], vraw[2][w], sel),
+                               __builtin_amdgcn_perm(vraw[5][w], vraw[4][w], sel),
+                               __builtin_amdgcn_perm(vraw[7][w], vraw[6][w], sel)};
           o[t] = Mma<E>::run(vf, pf, o[t]);
         }
         if (!more) break;
@@ -295,7 +246,7 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
   l_run += __shfl_xor(l_run, 32, kWave);
 
   // ---- merge the four waves: (2,3) -> LDS, (0,1) fold them in, 1 -> LDS, 0 folds and emits ----
-  auto spill = [&](int buf) {
+  auto spill = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < kDimTiles; ++t)
 #pragma unroll
@@ -305,7 +256,7 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
       ml_s[buf][j][1] = l_run;
     }
   };
-  auto fold = [&](int buf) {
+  auto fold = [&](int buf) __attribute__((always_inline)) {
     const float m_o = ml_s[buf][j][0], l_o = ml_s[buf][j][1];
     const float m_new = fmaxf(m_run, m_o);
     const float sa = exp2f(m_run - m_new), sb = exp2f(m_o - m_new);
@@ -359,6 +310,7 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
 
 template <typename E>
 static int launch_mfma_typed(const AttnArgs& a, int n_items, hipStream_t stream) {
+  if (n_items == 0) return VA_OK;
   const dim3 grid((unsigned)n_items, (unsigned)a.num_kv_heads), block(kMfmaThreads);
   switch (a.head_dim) {
     case 64:
@@ -377,7 +329,8 @@ static int launch_mfma_typed(const AttnArgs& a, int n_items, hipStream_t stream)
   return e == hipSuccess ? VA_OK : va_fail(VA_ERR_HIP, "attention launch: %s", hipGetErrorString(e));
 }
 
-int launch_mfma(const AttnArgs& a, int dtype, int n_items, int q_tile, hipStream_t stream) {
+int launch_mfma(const AttnArgs& a_in, int dtype, int n_items, int n_wide, int q_tile, hipStream_t stream) {
+  AttnArgs a = a_in;
   const int g = a.num_q_heads / a.num_kv_heads;
   if (!va_mfma_supported(dtype, a.head_dim, g))
     return va_fail(VA_ERR_ARG, "matrix-core path does not support this dtype/head_dim/group size");
@@ -385,7 +338,13 @@ int launch_mfma(const AttnArgs& a, int dtype, int n_items, int q_tile, hipStream
   if (a.rope.rotary_dim % 16) return va_fail(VA_ERR_ARG, "matrix-core path needs rotary_dim to be a multiple of 16");
   if (a.q_row_stride % 8 || a.pool_row_stride % 8)
     return va_fail(VA_ERR_ARG, "matrix-core path needs 16-byte aligned rows");
-  return dtype == VA_BF16 ? launch_mfma_typed<BF16>(a, n_items, stream) : launch_mfma_typed<F16>(a, n_items, stream);
+  if (n_wide > 0) {
+    const int rc = launch_mfma_wide(a, dtype, n_wide, stream);
+    if (rc) return rc;
+  }
+  a.items += (long long)n_wide * VA_ITEM_WORDS;
+  const int n_narrow = n_items - n_wide;
+  return dtype == VA_BF16 ? launch_mfma_typed<BF16>(a, n_narrow, stream) : launch_mfma_typed<F16>(a, n_narrow, stream);
 }
 
 }  // namespace va

@@ -1,0 +1,84 @@
+// Matrix-core helpers shared by the narrow and the wide attention kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "va_device.h"
+
+typedef __bf16 va_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 va_f16x8 __attribute__((ext_vector_type(8)));
+typedef float va_f32x4 __attribute__((ext_vector_type(4)));
+
+typedef float va_f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t va_u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes as a plain vector (registers, LDS)
+
+namespace va {
+
+template <typename E>
+struct Mma;
+template <>
+struct Mma<BF16> {
+  template <typename A, typename B>
+  static __device__ __forceinline__ va_f32x16 run32(const A& a, const B& b, va_f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(va_bf16x8, a), __builtin_bit_cast(va_bf16x8, b),
+                                                   c, 0, 0, 0);
+  }
+  template <typename A, typename B>
+  static __device__ __forceinline__ va_f32x4 run(const A& a, const B& b, va_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(va_bf16x8, a), __builtin_bit_cast(va_bf16x8, b),
+                                                   c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    const __bf16 l = (__bf16)lo, h = (__bf16)hi;
+    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+  }
+};
+template <>
+struct Mma<F16> {
+  template <typename A, typename B>
+  static __device__ __forceinline__ va_f32x16 run32(const A& a, const B& b, va_f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(va_f16x8, a), __builtin_bit_cast(va_f16x8, b), c,
+                                                  0, 0, 0);
+  }
+  template <typename A, typename B>
+  static __device__ __forceinline__ va_f32x4 run(const A& a, const B& b, va_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(va_f16x8, a), __builtin_bit_cast(va_f16x8, b), c,
+                                                  0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    const _Float16 l = (_Float16)lo, h = (_Float16)hi;
+    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+  }
+};
+
+// One 16-byte piece (dims [d0, d0+8)) of a query head row, rotated for position `p` and
+// rounded to the element type; pieces beyond rotary_dim pass through.  rotary_dim is a
+// multiple of 16 here, so a piece never straddles the two rotary halves.
+template <typename E>
+__device__ __forceinline__ uint4 rotated_query_piece(const RopeDev& rope, const typename E::storage* qh, int d0,
+                                                     const Pos3& p) {
+  using S = typename E::storage;
+  if (d0 >= rope.rotary_dim) return *(const uint4*)(qh + d0);
+  const bool first = d0 < rope.half;
+  const int i0 = first ? d0 : d0 - rope.half;
+  const uint4 ra = *(const uint4*)(qh + i0);
+  const uint4 rb = *(const uint4*)(qh + i0 + rope.half);
+  const uint32_t wa[4] = {ra.x, ra.y, ra.z, ra.w}, wb[4] = {rb.x, rb.y, rb.z, rb.w};
+  uint32_t out[4];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    float y[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const S xa = __builtin_bit_cast(S, (uint16_t)(wa[w] >> (16 * b)));
+      const S xb = __builtin_bit_cast(S, (uint16_t)(wb[w] >> (16 * b)));
+      float cs, sn, y1, y2;
+      rope_cos_sin(rope, p, i0 + 2 * w + b, cs, sn);
+      rope_pair<E>(rope, cs, sn, E::load(xa), E::load(xb), y1, y2);
+      y[b] = first ? y1 : y2;
+    }
+    out[w] = Mma<E>::pack(y[0], y[1]);  // y is already representable: the conversion is exact
+  }
+  return make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+}  // namespace va

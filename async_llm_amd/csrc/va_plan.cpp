@@ -29,7 +29,7 @@
 namespace {
 
 struct Item {
-  int32_t link_begin, n_links, n_q, part_base, tokens;
+  int32_t link_begin, n_links, n_q, part_base, tokens, kind;
 };
 struct Link {
   int32_t kv_begin, tok_begin, tok_end, qref, causal_base, flags;
@@ -43,7 +43,7 @@ struct Built {
   std::vector<int32_t> row_ids;
   std::vector<int32_t> row_flags;
   int32_t n_partials = 0;
-  int32_t kernel = 0, q_tile = 0, kv_chunk = 0;
+  int32_t kernel = 0, q_tile = 0, kv_chunk = 0, wide_tile = 0, n_wide = 0;
 };
 
 inline int32_t round_up(int64_t x, int32_t m) { return (int32_t)(((x + m - 1) / m) * m); }
@@ -106,6 +106,27 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   const bool has_chain = std::any_of(s->chain, s->chain + s->n_sub, [](int32_t c) { return c >= 0; });
   if (q_tile == 0) q_tile = kernel == VA_KERNEL_MFMA ? va_mfma_default_q_tile(g, has_chain) : 1;
   if (q_tile > q_tile_max) return va_fail(VA_ERR_ARG, "q_tile %d exceeds the kernel's maximum %d", q_tile, q_tile_max);
+  // Wide tiles (matrix-core path only): query tiles of more than q_tile rows are served by the
+  // wide kernel, whose four waves share every K/V tile through LDS.
+  int wide_tile = 0;
+  if (kernel == VA_KERNEL_MFMA && !(params && params->wide_tile < 0)) {
+    wide_tile = params && params->wide_tile > 0 ? params->wide_tile : va_mfma_wide_q_tile(g);
+    if (wide_tile > va_mfma_wide_q_tile(g))
+      return va_fail(VA_ERR_ARG, "wide_tile %d exceeds the kernel's maximum %d", wide_tile, va_mfma_wide_q_tile(g));
+    if (wide_tile <= q_tile) wide_tile = 0;
+  }
+  // Cut n query rows into tiles: wide ones while more than q_tile rows remain, then narrow ones.
+  auto cut_tiles = [&](int64_t n, std::vector<std::pair<int32_t, int32_t>>& tiles) {
+    tiles.clear();
+    int64_t a = 0;
+    while (a < n) {
+      const int64_t left = n - a;
+      const int64_t take = (wide_tile && left > q_tile) ? std::min<int64_t>(left, wide_tile) : std::min<int64_t>(left, q_tile);
+      tiles.emplace_back((int32_t)a, (int32_t)(a + take));
+      a += take;
+    }
+  };
+  std::vector<std::pair<int32_t, int32_t>> tiles;
   const int target = params && params->target_items > 0 ? params->target_items
                                                         : std::max(64, 2048 / shape->num_kv_heads);
   const int gran = 64;  // chunk boundaries are multiples of this many tokens
@@ -180,20 +201,18 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
 
   // ---- total tokens -> chunk size for split-KV ----
   int64_t total_tokens = 0;
-  int64_t n_group_tiles = 0;
   for (auto& gr : groups) {
-    const int64_t tiles = ((int64_t)gr.subrows.size() + q_tile - 1) / q_tile;
-    n_group_tiles += tiles;
-    total_tokens += tiles * s->seq_lens[gr.rep];
+    cut_tiles((int64_t)gr.subrows.size(), tiles);
+    total_tokens += (int64_t)tiles.size() * s->seq_lens[gr.rep];
   }
   int64_t chain_tiles = 0, chain_tokens = 0;
   for (auto& ch : chains) {
     const int32_t nq = s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]];
-    for (int32_t a = 0; a < nq; a += q_tile) {
-      const int32_t b = std::min(nq, a + q_tile);
+    cut_tiles(nq, tiles);
+    for (auto& tl : tiles) {
       ++chain_tiles;
       for (int32_t m : ch)
-        chain_tokens += visible_end(s->seq_lens[m], nq, s->flags[m] & VA_SUB_CAUSAL, b);
+        chain_tokens += visible_end(s->seq_lens[m], nq, s->flags[m] & VA_SUB_CAUSAL, tl.second);
     }
   }
   total_tokens += chain_tokens;
@@ -206,6 +225,7 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   out.kernel = kernel;
   out.q_tile = q_tile;
   out.kv_chunk = kv_chunk;
+  out.wide_tile = wide_tile;
 
   // contributions per output row decide direct-vs-partial
   std::vector<int32_t> row_count(s->n_rows, 0);
@@ -218,7 +238,7 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   auto emit = [&](int32_t n_q, const std::vector<Link>& links, std::vector<int32_t>&& rows) {
     int32_t tokens = 0;
     for (auto& l : links) tokens += l.tok_end - l.tok_begin;
-    Item it{(int32_t)out.links.size(), (int32_t)links.size(), n_q, -1, tokens};
+    Item it{(int32_t)out.links.size(), (int32_t)links.size(), n_q, -1, tokens, n_q > q_tile ? 1 : 0};
     out.links.insert(out.links.end(), links.begin(), links.end());
     for (int32_t r : rows) ++row_count[r];
     pend.push_back(Pending{(int32_t)out.items.size(), std::move(rows)});
@@ -231,8 +251,9 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     const int32_t n_chunks = (len + kv_chunk - 1) / kv_chunk;
     const int32_t per = round_up((len + n_chunks - 1) / n_chunks, gran);
     const int32_t lflags = VA_LINK_INDIRECT | ((s->flags[rep] & VA_SUB_SLOTS) ? VA_LINK_SLOTS : 0);
-    for (size_t a = 0; a < gr.subrows.size(); a += q_tile) {
-      const size_t b = std::min(gr.subrows.size(), a + (size_t)q_tile);
+    cut_tiles((int64_t)gr.subrows.size(), tiles);
+    for (auto& tl : tiles) {
+      const size_t a = tl.first, b = tl.second;
       const int32_t qref = (int32_t)out.qrefs.size();
       out.qrefs.insert(out.qrefs.end(), gr.subrows.begin() + a, gr.subrows.begin() + b);
       for (int32_t t0 = 0; t0 < len; t0 += per) {
@@ -257,8 +278,9 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   }
   for (auto& ch : chains) {
     const int32_t nq = s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]];
-    for (int32_t a = 0; a < nq; a += q_tile) {
-      const int32_t b = std::min(nq, a + q_tile);
+    cut_tiles(nq, tiles);
+    for (auto& tl : tiles) {
+      const int32_t a = tl.first, b = tl.second;
       std::vector<Link> all;
       int64_t tile_tokens = 0;
       for (int32_t m : ch) {
@@ -324,15 +346,21 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     else if (parts_of_row[r].empty()) out.row_flags[r] = VA_ROW_DIRECT;
   }
 
-  // longest items first: the tail of the launch is made of short items
+  // wide items first, then narrow ones; within a class longest first, so the tail of each
+  // launch is made of short items
   std::vector<int32_t> order(out.items.size());
   std::iota(order.begin(), order.end(), 0);
   std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) {
-    return (int64_t)out.items[x].tokens * out.items[x].n_q > (int64_t)out.items[y].tokens * out.items[y].n_q;
+    const Item &ix = out.items[x], &iy = out.items[y];
+    if (ix.kind != iy.kind) return ix.kind > iy.kind;
+    return (int64_t)ix.tokens * ix.n_q > (int64_t)iy.tokens * iy.n_q;
   });
   std::vector<Item> sorted;
   sorted.reserve(order.size());
-  for (int32_t i : order) sorted.push_back(out.items[i]);
+  for (int32_t i : order) {
+    sorted.push_back(out.items[i]);
+    out.n_wide += out.items[i].kind;
+  }
   out.items.swap(sorted);
   return VA_OK;
 }
@@ -341,6 +369,8 @@ void fill_counts(const Built& b, const VaSubRequests* s, const VaShape* shape, V
   c->kernel = b.kernel;
   c->q_tile = b.q_tile;
   c->kv_chunk = b.kv_chunk;
+  c->wide_tile = b.wide_tile;
+  c->n_wide_items = b.n_wide;
   c->n_items = (int32_t)b.items.size();
   c->n_links = (int32_t)b.links.size();
   c->n_qrefs = (int32_t)b.qrefs.size();
@@ -381,6 +411,8 @@ extern "C" int va_plan_build(const VaSubRequests* subs, const VaShape* shape, co
   h[VA_H_KERNEL] = c.kernel;
   h[VA_H_Q_TILE] = c.q_tile;
   h[VA_H_KV_CHUNK] = c.kv_chunk;
+  h[VA_H_N_WIDE] = c.n_wide_items;
+  h[VA_H_WIDE_TILE] = c.wide_tile;
   h[VA_H_N_ITEMS] = c.n_items;
   h[VA_H_N_LINKS] = c.n_links;
   h[VA_H_N_QREFS] = c.n_qrefs;
@@ -398,6 +430,7 @@ extern "C" int va_plan_build(const VaSubRequests* subs, const VaShape* shape, co
     w[VA_I_N_Q] = it.n_q;
     w[VA_I_PART_BASE] = it.part_base;
     w[VA_I_TOKENS] = it.tokens;
+    w[VA_I_KIND] = it.kind;
     off += VA_ITEM_WORDS;
   }
   h[VA_H_OFF_LINKS] = off;

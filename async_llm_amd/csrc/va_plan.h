@@ -33,6 +33,8 @@ enum {
   VA_H_OFF_ROW_FLAGS,
   VA_H_N_EMPTY_ROWS,   // rows no sub-request serves
   VA_H_N_SUBROWS,
+  VA_H_N_WIDE,     // items [0, n_wide) are wide tiles, the rest narrow
+  VA_H_WIDE_TILE,
 };
 
 // item word indices
@@ -42,6 +44,7 @@ enum {
   VA_I_N_Q,        // query rows in the tile
   VA_I_PART_BASE,  // first partial slot (one per query row), or -1: write `out` directly
   VA_I_TOKENS,     // KV tokens the item walks (scheduling weight)
+  VA_I_KIND,       // 1: wide tile (more rows than the narrow kernel's tile)
 };
 
 // link word indices

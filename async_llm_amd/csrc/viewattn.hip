@@ -510,7 +510,7 @@ extern "C" int va_attention(const void* q_dev, int64_t q_row_stride, const void*
 
   if (n_items > 0) {
     if (h[VA_H_KERNEL] == VA_KERNEL_MFMA) {
-      rc = va::launch_mfma(a, shape->dtype, n_items, h[VA_H_Q_TILE], s);
+      rc = va::launch_mfma(a, shape->dtype, n_items, h[VA_H_N_WIDE], h[VA_H_Q_TILE], s);
     } else {
       VA_DISPATCH_DTYPE(shape->dtype, rc = va::launch_generic<E>(a, n_items, s));
     }

@@ -78,6 +78,7 @@ class VaPlanParams(C.Structure):
         ("q_tile", C.c_int32),
         ("kv_chunk", C.c_int32),
         ("target_items", C.c_int32),
+        ("wide_tile", C.c_int32),
     ]
 
 
@@ -92,6 +93,8 @@ class VaPlanCounts(C.Structure):
         ("n_partials", C.c_int32),
         ("n_row_parts", C.c_int32),
         ("plan_words", C.c_int32),
+        ("wide_tile", C.c_int32),
+        ("n_wide_items", C.c_int32),
         ("workspace_bytes", C.c_int64),
     ]
 

@@ -167,7 +167,7 @@ class SharedCacheAttention:
         if kernel == "auto" and self.rotary_dim % 16:
             kernel = "generic"  # the matrix-core kernel rotates queries in 8-element pieces
         self.kernel = kernel
-        self.plan_params = native.VaPlanParams(_KERNELS[kernel], 0, 0, 0)
+        self.plan_params = native.VaPlanParams(_KERNELS[kernel], 0, 0, 0, 0)
         self._shape = native.make_shape(num_qo_heads, num_kv_heads, head_dim, page_size, dtype)
         self._rope_desc: Optional[native.VaRope] = None
         self._workspace: Optional[torch.Tensor] = None

@@ -140,6 +140,7 @@ typedef struct VaPlanParams {
   int32_t q_tile;        /* 0 = library default for the chosen kernel         */
   int32_t kv_chunk;      /* 0 = derive from the launch's total KV tokens      */
   int32_t target_items;  /* 0 = default (work items wanted per kv head)       */
+  int32_t wide_tile;     /* rows of a wide query tile: 0 = default, <0 = never */
 } VaPlanParams;
 
 typedef struct VaPlanCounts {
@@ -152,6 +153,8 @@ typedef struct VaPlanCounts {
   int32_t n_partials;    /* partial (row, item) slots the launch will write */
   int32_t n_row_parts;   /* length of row_part_ids */
   int32_t plan_words;    /* int32 words va_plan_build writes                 */
+  int32_t wide_tile;     /* resolved rows of a wide tile (0: none)           */
+  int32_t n_wide_items;  /* items served by the wide kernel                  */
   int64_t workspace_bytes; /* device scratch va_attention needs for this plan */
 } VaPlanCounts;
 

@@ -15,7 +15,7 @@ from async_llm_amd import native
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 H = dict(MAGIC=0, KERNEL=1, Q_TILE=2, KV_CHUNK=3, N_ITEMS=4, N_LINKS=5, N_QREFS=6, N_PARTIALS=7, N_ROW_PARTS=8,
          N_ROWS=9, OFF_ITEMS=10, OFF_LINKS=11, OFF_QREFS=12, OFF_ROW_INDPTR=13, OFF_ROW_IDS=14, OFF_ROW_FLAGS=15,
-         N_EMPTY=16, N_SUBROWS=17)
+         N_EMPTY=16, N_SUBROWS=17, N_WIDE=18, WIDE_TILE=19)
 NO_CAUSAL = 0x3FFFFFFF
 
 
@@ -32,14 +32,14 @@ def test_library_exports_every_declared_symbol():
 
 
 def build_plan(qo, kvp, kvi, lens, flags, chain, sub_worker, n_rows, heads=(8, 2, 64), page=4, dtype=native.VA_F32,
-               kernel=native.VA_KERNEL_GENERIC, q_tile=0, kv_chunk=0, target=0):
+               kernel=native.VA_KERNEL_GENERIC, q_tile=0, kv_chunk=0, target=0, wide_tile=0):
     arr = [np.ascontiguousarray(a, dtype=np.int32) for a in (qo, kvp, kvi, lens, flags, chain)]
     sw = np.ascontiguousarray(sub_worker, dtype=np.int64)
     subs = native.VaSubRequests(len(lens), len(sw), n_rows, arr[0].ctypes.data, arr[1].ctypes.data,
                                 arr[2].ctypes.data if arr[2].size else None, arr[3].ctypes.data,
                                 arr[4].ctypes.data, arr[5].ctypes.data, sw.ctypes.data if sw.size else None)
     shape = native.VaShape(heads[0], heads[1], heads[2], page, dtype)
-    params = native.VaPlanParams(kernel, q_tile, kv_chunk, target)
+    params = native.VaPlanParams(kernel, q_tile, kv_chunk, target, wide_tile)
     counts = native.VaPlanCounts()
     rc = native.lib.va_plan_count(subs, shape, params, counts)
     if rc:
@@ -76,7 +76,8 @@ def check_coverage(blob, qo, kvp, lens, flags, sub_worker, n_rows):
     contributions = [0] * n_rows
     for it in items:
         lb, nl, nq, part_base = it[0], it[1], it[2], it[3]
-        assert nl >= 1 and 1 <= nq <= h[H["Q_TILE"]]
+        assert nl >= 1 and 1 <= nq <= max(h[H["Q_TILE"]], h[H["WIDE_TILE"]])
+        assert it[5] == int(nq > h[H["Q_TILE"]])  # kind: wide iff more rows than the narrow tile
         rows_of_item = None
         for l in links[lb: lb + nl]:
             kv_begin, t0, t1, qref, cbase, lflags = l[:6]
@@ -185,6 +186,26 @@ def test_plan_covers_every_visible_pair_once(seed, prefill, q_tile, kv_chunk, ta
     check_coverage(blob, qo, kvp, lens, flags, sub_worker, n_rows)
 
 
+@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("prefill", [False, True])
+@pytest.mark.parametrize("wide_tile", [0, 8, -1])
+def test_matrix_core_plans_with_wide_tiles_cover_every_pair_once(seed, prefill, wide_tile):
+    rng = random.Random(100 + seed * 2 + int(prefill))
+    page = rng.choice([1, 4, 16])
+    qo, kvp, kvi, lens, flags, chain, sub_worker, n_rows = random_tables(rng, page, prefill)
+    rc, blob, counts = build_plan(qo, kvp, kvi, lens, flags, chain, sub_worker, n_rows, page=page, dtype=native.VA_BF16,
+                                  kernel=native.VA_KERNEL_MFMA, wide_tile=wide_tile, kv_chunk=rng.choice([0, 64]))
+    assert rc == 0, native.lib.va_last_error()
+    assert counts.kernel == native.VA_KERNEL_MFMA and counts.q_tile == 4
+    assert counts.wide_tile == {0: 32, 8: 8, -1: 0}[wide_tile]
+    h, items, *_ = decode_plan(blob)
+    kinds = [int(i[5]) for i in items]
+    assert kinds == sorted(kinds, reverse=True) and sum(kinds) == counts.n_wide_items == h[H["N_WIDE"]]
+    if wide_tile < 0:
+        assert counts.n_wide_items == 0
+    check_coverage(blob, qo, kvp, lens, flags, sub_worker, n_rows)
+
+
 def test_readers_of_one_block_share_a_tile():
     page, L = 4, 300
     pages = list(range(75))
@@ -225,7 +246,7 @@ def test_plan_rejects_inconsistent_tables():
     sw = np.ascontiguousarray(ok["sub_worker"], dtype=np.int64)
     subs = native.VaSubRequests(1, 1, 1, a[0].ctypes.data, a[1].ctypes.data, a[2].ctypes.data, a[3].ctypes.data,
                                 a[4].ctypes.data, a[5].ctypes.data, sw.ctypes.data)
-    rc = native.lib.va_plan_build(subs, native.VaShape(8, 2, 64, 4, 0), native.VaPlanParams(1, 0, 0, 0),
+    rc = native.lib.va_plan_build(subs, native.VaShape(8, 2, 64, 4, 0), native.VaPlanParams(1, 0, 0, 0, 0),
                                   subs_blob.ctypes.data, 4, None)
     assert rc == -2 and "words" in native.lib.va_last_error().decode()
 
