@@ -112,6 +112,8 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     // tokens any row of this wave sees (none if the wave's rows lie beyond the tile)
     const int t_wave = (32 * wave) / G < n_q ? min(tok_end, causal_base + wave_iq_last + 1) : -0x7fffffff;
     const int t_last = t_stop - 1;
+    // tokens EVERY real row of this wave sees: tiles ending below it need no masking
+    const int t_wave_min = min(tok_end, causal_base + (32 * wave) / G + 1);
 
     // global -> registers -> LDS.  Thread (ld_tok, ld_c) moves piece ld_c of tokens ld_tok + kTokStep*i of
     // both the K and the V tile: rows are contiguous over threads, K and V share the row lookup.
@@ -183,30 +185,51 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
 #endif
         const va_u32x4* kt = k_tile(buf);
         const va_u32x4* vt = v_tile(buf);
-        // ---- scores ----
+        // ---- scores.  K fragments are read from LDS in groups of four, two groups ahead of the
+        // MFMAs that consume them, so the matrix pipe never waits on an LDS round trip. ----
+        constexpr int kGroups = kSteps / 4;
+        va_u32x4 kfr[2][4];
+        auto read_group = [&](int g, va_u32x4 (&dst)[4]) __attribute__((always_inline)) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) dst[q] = kt[j * kRow + 2 * (4 * g + q) + h];
+        };
+        read_group(0, kfr[0]);
+        if constexpr (kGroups > 1) read_group(1, kfr[1]);
         va_f32x16 sc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+        __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs (the scheduler would sink them)
 #pragma unroll
-        for (int s = 0; s < kSteps; ++s) sc = Mma<E>::run32(kt[j * kRow + 2 * s + h], qf[s], sc);
+        for (int g = 0; g < kGroups; ++g) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) sc = Mma<E>::run32(kfr[g & 1][q], qf[4 * g + q], sc);
+          if (g + 2 < kGroups) read_group(g + 2, kfr[g & 1]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
 
-        // ---- online softmax: reg r holds token t0 + (r/4)*8 + 4h + r%4 of row my_row ----
+        // ---- online softmax: reg r holds token t0 + (r/4)*8 + 4h + r%4 of row my_row.  Interior
+        // tiles (every row of the wave sees all 32 tokens) skip the masking; the scale is folded
+        // into the exponent: p = 2^(s*c - m). ----
         float tile_max = -INFINITY;
+        if (t0 + kWideTokens <= t_wave_min) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int t = t0 + (r / 4) * 8 + 4 * h + (r % 4);
-          const float v = t < t_row ? sc[r] * a.scale_log2 : -INFINITY;
-          sc[r] = v;
-          tile_max = fmaxf(tile_max, v);
+          for (int r = 0; r < 16; ++r) tile_max = fmaxf(tile_max, sc[r]);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int t = t0 + (r / 4) * 8 + 4 * h + (r % 4);
+            sc[r] = t < t_row ? sc[r] : -INFINITY;
+            tile_max = fmaxf(tile_max, sc[r]);
+          }
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
-        const float m_new = fmaxf(m_run, tile_max);
-        const float alpha = exp2f(m_run - m_new);
+        const float m_new = fmaxf(m_run, tile_max * a.scale_log2);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         m_run = m_new;
         float psum = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          sc[r] = exp2f(sc[r] - m_new);
+          sc[r] = __builtin_amdgcn_exp2f(fmaf(sc[r], a.scale_log2, -m_new));
           psum += sc[r];
         }
         l_run = l_run * alpha + psum;

@@ -116,17 +116,21 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     if (wide_tile <= q_tile) wide_tile = 0;
   }
   // Cut n query rows into tiles: wide ones while more than q_tile rows remain, then narrow ones.
-  auto cut_tiles = [&](int64_t n, std::vector<std::pair<int32_t, int32_t>>& tiles) {
+  auto cut_tiles = [&](int64_t n, std::vector<std::pair<int32_t, int32_t>>& tiles, bool allow_wide = true) {
     tiles.clear();
     int64_t a = 0;
     while (a < n) {
       const int64_t left = n - a;
-      const int64_t take = (wide_tile && left > q_tile) ? std::min<int64_t>(left, wide_tile) : std::min<int64_t>(left, q_tile);
+      const int64_t take = (allow_wide && wide_tile && left > q_tile) ? std::min<int64_t>(left, wide_tile) : std::min<int64_t>(left, q_tile);
       tiles.emplace_back((int32_t)a, (int32_t)(a + take));
       a += take;
     }
   };
   std::vector<std::pair<int32_t, int32_t>> tiles;
+  // Decode groups (readers of one shared block) use wide tiles only on request: at decode sizes the
+  // extra launch costs more than the re-reads it saves; their narrow tiles are emitted chunk-major
+  // instead, so the tiles that stream the same chunk run side by side and share it in L2.
+  const bool wide_groups = params && params->wide_tile > 0;
   const int target = params && params->target_items > 0 ? params->target_items
                                                         : std::max(64, 2048 / shape->num_kv_heads);
   const int gran = 64;  // chunk boundaries are multiples of this many tokens
@@ -202,7 +206,7 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   // ---- total tokens -> chunk size for split-KV ----
   int64_t total_tokens = 0;
   for (auto& gr : groups) {
-    cut_tiles((int64_t)gr.subrows.size(), tiles);
+    cut_tiles((int64_t)gr.subrows.size(), tiles, wide_groups);
     total_tokens += (int64_t)tiles.size() * s->seq_lens[gr.rep];
   }
   int64_t chain_tiles = 0, chain_tokens = 0;
@@ -245,25 +249,47 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     out.items.push_back(it);
   };
 
+  // Wide decode tiles run in their own launch (one workgroup per CU at a time), so their
+  // runs are cut finer: enough chunks for about one workgroup per CU.
+  int64_t wide_group_tokens = 0;
+  for (auto& gr : groups) {
+    cut_tiles((int64_t)gr.subrows.size(), tiles, wide_groups);
+    for (auto& tl : tiles)
+      if (tl.second - tl.first > q_tile) wide_group_tokens += s->seq_lens[gr.rep];
+  }
+  const int wide_items_wanted = std::max(1, 256 / shape->num_kv_heads);
+  const int32_t wide_chunk = std::min<int32_t>(
+      kv_chunk, round_up(std::max<int64_t>((wide_group_tokens + wide_items_wanted - 1) / wide_items_wanted, 2 * gran), gran));
+
   for (auto& gr : groups) {
     const int32_t rep = gr.rep;
     const int32_t len = s->seq_lens[rep];
-    const int32_t n_chunks = (len + kv_chunk - 1) / kv_chunk;
-    const int32_t per = round_up((len + n_chunks - 1) / n_chunks, gran);
     const int32_t lflags = VA_LINK_INDIRECT | ((s->flags[rep] & VA_SUB_SLOTS) ? VA_LINK_SLOTS : 0);
-    cut_tiles((int64_t)gr.subrows.size(), tiles);
+    cut_tiles((int64_t)gr.subrows.size(), tiles, wide_groups);
+    std::vector<int32_t> tile_qref;
     for (auto& tl : tiles) {
-      const size_t a = tl.first, b = tl.second;
-      const int32_t qref = (int32_t)out.qrefs.size();
-      out.qrefs.insert(out.qrefs.end(), gr.subrows.begin() + a, gr.subrows.begin() + b);
-      for (int32_t t0 = 0; t0 < len; t0 += per) {
-        std::vector<int32_t> rows;
-        for (size_t r = a; r < b; ++r) rows.push_back((int32_t)s->sub_worker[gr.subrows[r]]);
-        emit((int32_t)(b - a),
-             {Link{s->kv_indptr[rep], t0, std::min(len, t0 + per), qref, VA_NO_CAUSAL, lflags}},
-             std::move(rows));
-      }
+      tile_qref.push_back((int32_t)out.qrefs.size());
+      out.qrefs.insert(out.qrefs.end(), gr.subrows.begin() + tl.first, gr.subrows.begin() + tl.second);
     }
+    auto emit_range = [&](size_t ti, int32_t t0, int32_t t1) {
+      const size_t a = tiles[ti].first, b = tiles[ti].second;
+      std::vector<int32_t> rows;
+      for (size_t r = a; r < b; ++r) rows.push_back((int32_t)s->sub_worker[gr.subrows[r]]);
+      emit((int32_t)(b - a), {Link{s->kv_indptr[rep], t0, t1, tile_qref[ti], VA_NO_CAUSAL, lflags}}, std::move(rows));
+    };
+    auto chunk_len = [&](int32_t chunk) {
+      const int32_t n_chunks = (len + chunk - 1) / chunk;
+      return round_up((len + n_chunks - 1) / n_chunks, gran);
+    };
+    // narrow tiles: chunk-major; wide tiles: their own (finer) chunking
+    const int32_t per = chunk_len(kv_chunk);
+    for (int32_t t0 = 0; t0 < len; t0 += per)
+      for (size_t ti = 0; ti < tiles.size(); ++ti)
+        if (tiles[ti].second - tiles[ti].first <= q_tile) emit_range(ti, t0, std::min(len, t0 + per));
+    const int32_t per_w = chunk_len(wide_chunk);
+    for (size_t ti = 0; ti < tiles.size(); ++ti)
+      if (tiles[ti].second - tiles[ti].first > q_tile)
+        for (int32_t t0 = 0; t0 < len; t0 += per_w) emit_range(ti, t0, std::min(len, t0 + per_w));
   }
 
   // chains are split only when tiles alone cannot fill the machine
