@@ -69,7 +69,7 @@ class SharedCacheAttnMetadata(BaseAttnMetadata):
     n_aux: int = 0  # decode: single-slot sub-requests (writer outside its own view)
     n_ctx_rows: int = 0  # prefill: sub-rows of the non-causal context part
     last_indices: Optional[torch.Tensor] = None
-    phase: Literal["decode", "prefill_batch"] = "decode"
+    phase: Literal["decode", "prefill_batch", "mixed"] = "decode"
     _plan_refs: tuple = field(default=(), repr=False)
     graph_buffers: object | None = field(default=None, repr=False)
     # host copies of the planned tables, keyed like the reference's FlashInfer plan() kwargs
@@ -78,7 +78,7 @@ class SharedCacheAttnMetadata(BaseAttnMetadata):
     launch: Optional[LaunchPlan] = field(default=None, repr=False)
 
     def get_last_indices(self, bs: int) -> torch.Tensor:
-        if self.phase == "prefill_batch":
+        if self.phase in ("prefill_batch", "mixed"):
             assert self.last_indices is not None
             return self.last_indices
         return torch.arange(bs, device=self.sub_worker.device)
@@ -248,20 +248,9 @@ class SharedCacheAttention:
         header = host[: native.PLAN_HEADER_WORDS].numpy().copy()
         return LaunchPlan(header, blob, kv_indices_dev, counts, self._ensure_workspace(counts.workspace_bytes))
 
-    def prepare(
-        self,
-        group,
-        new_page_for_block: Dict[int, Optional[int]],
-        new_token_slots: torch.Tensor,
-        graph_buffers=None,
-    ) -> SharedCacheAttnMetadata:
-        """Plan one decode step (reference ``attention.py:282-448``).
-
-        ``new_page_for_block`` maps ``id(write_block)`` to the page-start slot of
-        the page this step's token opens (``None`` if it fits the last page); its
-        keys are the blocks written this step.  ``new_token_slots [W]`` are the
-        slots of the new tokens.  Blocks are not modified.
-        """
+    def _walk_decode(self, group, new_page_for_block, new_token_slots):
+        """Sub-requests of one decode step: per worker one paged sub-request per
+        non-empty view block, plus a single-slot one when it writes outside its view."""
         W = group.num_workers
         assert W > 0
         P = self.page_size
@@ -303,6 +292,26 @@ class SharedCacheAttention:
                 aux["kv"].append(slots_host[w])
                 seg += 1
             max_segments = max(max_segments, seg)
+
+        return main, aux, max_segments
+
+    def prepare(
+        self,
+        group,
+        new_page_for_block: Dict[int, Optional[int]],
+        new_token_slots: torch.Tensor,
+        graph_buffers=None,
+    ) -> SharedCacheAttnMetadata:
+        """Plan one decode step (reference ``attention.py:282-448``).
+
+        ``new_page_for_block`` maps ``id(write_block)`` to the page-start slot of
+        the page this step's token opens (``None`` if it fits the last page); its
+        keys are the blocks written this step.  ``new_token_slots [W]`` are the
+        slots of the new tokens.  Blocks are not modified.
+        """
+        W = group.num_workers
+        P = self.page_size
+        main, aux, max_segments = self._walk_decode(group, new_page_for_block, new_token_slots)
 
         if graph_buffers is not None:
             return graph_buffers.plan(main["worker"], main["loc"], main["slot"], main["pages"], main["n_pages"],
@@ -360,17 +369,10 @@ class SharedCacheAttention:
         refs.extend((host, dev))
         return [dev[i] for i in range(len(rows))]
 
-    def prepare_prefill_batch(self, specs: List[PrefillSpec], graph_buffers=None) -> SharedCacheAttnMetadata:
-        """Plan several view-conditioned prefills as one launch, request-major
-        (reference ``attention.py:450-622``).  Request ``r`` owns output rows
-        ``[offset_r, offset_r + num_new_r)``; its new tokens attend fully to each
-        context block (sized before this step's writes) and causally to their
-        own block, prefix included."""
-        assert specs, "prepare_prefill_batch needs at least one request"
-        if graph_buffers is not None:
-            return graph_buffers.plan(specs)
+    def _walk_prefill(self, specs, use_3d: bool):
+        """Sub-requests of a batched prefill: per request one non-causal sub-request
+        per context block and one causal sub-request over its own block."""
         P = self.page_size
-        use_3d = any(s.mrope_rel is not None for s in specs)
         max_segments = max(len(s.context) + 1 for s in specs)
         snapshot: Dict[int, List[int]] = {}
 
@@ -414,6 +416,21 @@ class SharedCacheAttention:
             own["chain"].append(r)
             last_indices.append(offset + S - 1)
             offset += S
+
+        return ctx, own, last_indices, offset, max_segments
+
+    def prepare_prefill_batch(self, specs: List[PrefillSpec], graph_buffers=None) -> SharedCacheAttnMetadata:
+        """Plan several view-conditioned prefills as one launch, request-major
+        (reference ``attention.py:450-622``).  Request ``r`` owns output rows
+        ``[offset_r, offset_r + num_new_r)``; its new tokens attend fully to each
+        context block (sized before this step's writes) and causally to their
+        own block, prefix included."""
+        assert specs, "prepare_prefill_batch needs at least one request"
+        if graph_buffers is not None:
+            return graph_buffers.plan(specs)
+        P = self.page_size
+        use_3d = any(s.mrope_rel is not None for s in specs)
+        ctx, own, last_indices, offset, max_segments = self._walk_prefill(specs, use_3d)
 
         n_rows = offset
         sub_gather = np.concatenate(ctx["rows"] + own["rows"])
@@ -464,6 +481,73 @@ class SharedCacheAttention:
             num_workers=n_rows, max_segments=max_segments, n_ctx_rows=n_ctx_rows,
             last_indices=to_dev(torch.tensor(last_indices, dtype=torch.int64)),
             phase="prefill_batch", main_plan=ctx_plan, aux_plan=self_plan, launch=launch)
+        meta._plan_refs = tuple(refs)
+        return meta
+
+    def prepare_mixed(self, group, new_page_for_block: Dict[int, Optional[int]], new_token_slots: torch.Tensor,
+                      specs: List[PrefillSpec]) -> SharedCacheAttnMetadata:
+        """Plan one decode step AND a batch of view-conditioned prefill chunks as a
+        single launch (a continuous batch).  Output rows are the ``W`` decode
+        workers followed by the prefill tokens, request-major; ``forward`` takes
+        q/k/v, ``positions`` and ``out_loc`` in that row order.  The two parts
+        keep their own semantics (``prepare`` / ``prepare_prefill_batch``): all new
+        K/V rows are stored before any attention runs, decode lengths count this
+        step's decode appends, prefill context lengths are pre-write.  The
+        reference runs the two as separate forwards (``session.decode_step`` /
+        ``prefill_batch``); nothing in its tables changes, they are concatenated.
+        """
+        assert specs, "prepare_mixed needs at least one prefill request (use prepare otherwise)"
+        W = group.num_workers
+        assert W > 0
+        P = self.page_size
+        use_3d = any(s.mrope_rel is not None for s in specs)
+        main, aux, seg_d = self._walk_decode(group, new_page_for_block, new_token_slots)
+        ctx, own, last_indices, n_new, seg_p = self._walk_prefill(specs, use_3d)
+        M = max(seg_d, seg_p)
+        n_main, n_aux, n_ctx, n_self = len(main["worker"]), len(aux["worker"]), len(ctx["q"]), len(own["q"])
+
+        refs: List[torch.Tensor] = []
+        parts = list(main["pages"]) + ([aux["kv"]] if n_aux else []) + ctx["pages"] + own["pages"]
+        kv_indices = upload_page_indices(parts, self.device, refs)
+        kv_host = refs[0]
+        kv_counts = main["n_pages"] + [1] * n_aux + ctx["n_pages"] + own["n_pages"]
+
+        dec_worker = np.asarray(main["worker"] + aux["worker"], dtype=np.int64)
+        dec_slot = np.asarray(main["slot"] + aux["slot"], dtype=np.int64)
+        dec_loc = torch.tensor(main["loc"] + aux["loc"], dtype=torch.int64)
+        pre_rows = np.concatenate(ctx["rows"] + own["rows"]) + W
+        pre_slot = np.concatenate(ctx["slot"] + own["slot"])
+        pre_loc = torch.cat(ctx["loc"] + own["loc"], dim=1 if use_3d else 0)
+        if use_3d:
+            dec_loc = dec_loc.unsqueeze(0).expand(3, -1)
+        sub_worker = np.concatenate([dec_worker, pre_rows])
+        sub_loc = torch.cat([dec_loc, pre_loc], dim=1 if use_3d else 0)
+        pad_slot = sub_worker * M + np.concatenate([dec_slot, pre_slot])
+
+        launch = self._build_launch(
+            qo_indptr=np.cumsum([0] + [1] * (n_main + n_aux) + ctx["q"] + own["q"]),
+            kv_indptr=np.cumsum([0] + kv_counts),
+            kv_indices_host=kv_host.numpy(),
+            seq_lens=main["len"] + [1] * n_aux + ctx["len"] + own["len"],
+            flags=[0] * n_main + [native.VA_SUB_SLOTS] * n_aux + [0] * n_ctx + [native.VA_SUB_CAUSAL] * n_self,
+            chain=[-1] * (n_main + n_aux) + ctx["chain"] + own["chain"],
+            sub_worker_host=sub_worker,
+            n_rows=W + n_new, kv_indices_dev=kv_indices, refs=refs)
+
+        def to_dev(t: torch.Tensor) -> torch.Tensor:
+            host = t.contiguous()
+            if self.device.type == "cuda":
+                host = host.pin_memory()
+            dev = host.to(self.device, non_blocking=True)
+            refs.extend((host, dev))
+            return dev
+
+        last = torch.cat([torch.arange(W, dtype=torch.int64), torch.tensor(last_indices, dtype=torch.int64) + W])
+        meta = SharedCacheAttnMetadata(
+            shared_cache_op=self, sub_worker=to_dev(torch.from_numpy(sub_worker)), sub_loc=to_dev(sub_loc),
+            pad_slot=to_dev(torch.from_numpy(pad_slot)), num_workers=W + n_new, max_segments=M,
+            n_main=n_main, n_aux=n_aux, n_ctx_rows=int(sum(ctx["q"])), last_indices=to_dev(last),
+            phase="mixed", launch=launch)
         meta._plan_refs = tuple(refs)
         return meta
 

@@ -275,3 +275,74 @@ def view_prefill(device, requests: int = 8, new_tokens: int = 2048, own_prefix: 
     return Workload("view_prefill", "prefill", op, pool, q, k, v, batch, [prompt] + own, theta, specs=specs,
                     alg_bytes=alg_bytes, logical_bytes=b_tok * pairs // max(1, new_tokens),
                     alg_flops=4 * D * Hq * pairs, info=dict(rows=N, visible_pairs=pairs))
+
+
+def mixed_batch(device, decode_rows: int = 48, chunks: int = 4, chunk_len: int = 512, ctx_lo: int = 1024,
+                ctx_hi: int = 32768, shared_len: int = 512, layers: int = 1, heads=(16, 4, 256),
+                dtype=torch.bfloat16, page_size: int = 16, seed: int = 3, kernel: Optional[str] = None) -> Workload:
+    """Configuration 4: a continuous batch in ONE launch -- ``decode_rows`` decode
+    requests plus ``chunks`` prefill chunks of ``chunk_len`` tokens.  Every view
+    starts with the shared prompt block and has 2-5 blocks in total; the total
+    context per row is uniform in [ctx_lo, ctx_hi] and split over the private
+    blocks by a seeded random composition (every block >= 16 tokens).  Decode rows
+    append to their last block; a chunk row extends its last block (the block's
+    current length is the chunk's prefix) and reads the blocks before it."""
+    Hq, Hkv, D = heads
+    P, theta = page_size, 1e7
+    gen = torch.Generator().manual_seed(seed)
+    rows = decode_rows + chunks
+    totals = torch.randint(ctx_lo, ctx_hi + 1, (rows,), generator=gen).tolist()
+    counts = torch.randint(2, 6, (rows,), generator=gen).tolist()
+    splits = []
+    for total, n in zip(totals, counts):
+        rest, parts = max(total - shared_len, 16 * (n - 1)), n - 1
+        w = torch.rand(parts, generator=gen)
+        extra = ((rest - 16 * parts) * w / w.sum()).floor().to(torch.int64).tolist()
+        lens = [16 + e for e in extra]
+        lens[-1] += rest - sum(lens)
+        splits.append(lens)
+    need = -(-shared_len // P) + sum(-(-n // P) + 1 for ls in splits for n in ls) + chunks * (chunk_len // P + 2) + rows
+    pages = _Pages(need, P, gen)
+    pool = _make_pool(Hkv, D, need, P, dtype, device, layers, seed, 1.0)
+    op = SharedCacheAttention(pool, build_cos_sin_cache(D, ctx_hi + chunk_len + shared_len + 64, theta, device), Hq, Hkv, D,
+                              P, dtype, device, kernel=kernel)
+    shared = _filled_block(pages, device, P, shared_len)
+    blocks, views, write_to, specs = [shared], [], [], []
+    positions, out_loc = [], []
+    pairs = 0
+    for r, ls in enumerate(splits):
+        mine = [_filled_block(pages, device, P, n) for n in ls]
+        blocks += mine
+        if r < decode_rows:
+            views.append([shared] + mine)
+            write_to.append(mine[-1])
+        else:
+            own, context = mine[-1], [shared] + mine[:-1]
+            fresh = pages.take(own.pages_needed(chunk_len))
+            starts = torch.tensor(own.page_starts + fresh, dtype=torch.int32)
+            specs.append(PrefillSpec(context, starts, chunk_len, own.num_tokens))
+            slots = (starts[:, None] + torch.arange(P, dtype=torch.int32)[None, :]).reshape(-1)
+            out_loc.append(slots[own.num_tokens:own.num_tokens + chunk_len])
+            positions.append(torch.arange(own.num_tokens, own.num_tokens + chunk_len, dtype=torch.int64))
+            pairs += chunk_len * (sum(b.num_tokens for b in context) + own.num_tokens) + chunk_len * (chunk_len + 1) // 2
+    group = WorkerGroup(cache_structure=views, write_to=write_to)
+    pending, slots_d, write_pos = plan_decode_writes(group, P, pages, device)
+    meta = op.prepare_mixed(group, pending, slots_d, specs)
+    N = decode_rows + chunks * chunk_len
+    q = torch.randn(N, Hq * D, generator=gen).to(dtype).to(device)
+    k = torch.randn(N, Hkv * D, generator=gen).to(dtype).to(device)
+    v = torch.randn(N, Hkv * D, generator=gen).to(dtype).to(device)
+    batch = SimpleNamespace(
+        attn_metadata=meta,
+        positions=torch.cat([torch.tensor(write_pos, dtype=torch.int64)] + positions).to(device),
+        out_loc=torch.cat([slots_d.cpu()] + out_loc).to(device), mrope_positions=None)
+    item = q.element_size()
+    b_tok = 2 * Hkv * D * item
+    distinct = sum(b.num_tokens for b in blocks) + decode_rows + chunks * chunk_len
+    logical = sum(sum(b.num_tokens for b in view) + 1 for view in views)
+    alg_bytes = b_tok * distinct + 2 * N * Hq * D * item + 4 * N * Hq + 4 * meta.launch.kv_indices.numel() + N * b_tok
+    return Workload("mixed_batch", "mixed", op, pool, q, k, v, batch, blocks, theta, group=group, pending=pending,
+                    new_token_slots=slots_d, specs=specs, alg_bytes=alg_bytes, logical_bytes=b_tok * logical,
+                    alg_flops=4 * D * Hq * (pairs + logical),
+                    info=dict(rows=N, decode_rows=decode_rows, chunks=chunks, chunk_len=chunk_len,
+                              prefill_pairs=pairs))

@@ -89,3 +89,37 @@ def test_scaled_view_prefill_configuration(kernel):
     pairs = 3 * (96 * (300 + 2 * 40) + 96 * 40 + 96 * 97 // 2)
     assert wl.alg_flops == 4 * D * Hq * pairs
     assert wl.meta.last_indices.tolist() == [95, 191, 287]
+
+
+@pytest.mark.parametrize("kernel", KERNELS)
+def test_mixed_batch_single_launch(kernel):
+    """Configuration 4 at reduced size: decode rows and prefill chunks planned and
+    run as ONE launch; each part must equal its own oracle evaluation over the
+    pool after ALL new rows were stored."""
+    from tests.util import oracle_decode_plan
+
+    wl = workloads.mixed_batch(DEV, decode_rows=5, chunks=2, chunk_len=40, ctx_lo=100, ctx_hi=900, shared_len=70,
+                               kernel=kernel)
+    op, meta = wl.op, wl.meta
+    Hq, Hkv, D, P = op.num_qo_heads, op.num_kv_heads, op.head_dim, op.page_size
+    W, N = 5, 5 + 2 * 40
+    assert meta.phase == "mixed" and meta.num_workers == N
+    assert meta.get_last_indices(0).tolist() == [0, 1, 2, 3, 4, 5 + 39, 5 + 79]
+    assert len(set(meta.pad_slot.tolist())) == meta.pad_slot.numel()
+    k_cpu, v_cpu = wl.pool.k_cache(0).cpu(), wl.pool.v_cache(0).cpu()
+    out, lse = op.forward_with_lse(wl.q, wl.k, wl.v, 0, wl.batch)
+    rope = oracle_rope(op, wl.theta)
+    k_rot = rope.rotate(wl.k.cpu().view(N, Hkv, D), wl.batch.positions.cpu())
+    O.store_kv(k_cpu.view(-1, Hkv * D), v_cpu.view(-1, Hkv * D), wl.batch.out_loc.cpu(), k_rot.reshape(N, -1), wl.v.cpu())
+    assert torch.equal(wl.pool.k_cache(0).cpu(), k_cpu) and torch.equal(wl.pool.v_cache(0).cpu(), v_cpu)
+    dplan = oracle_decode_plan(wl.group, wl.pending, wl.new_token_slots.cpu(), P)
+    pplan = oracle_prefill_plan(wl.specs, P)
+    assert meta.sub_loc.tolist() == dplan.sub_loc + pplan.sub_loc.tolist()
+    assert meta.sub_worker.tolist() == dplan.sub_worker + [r + W for r in pplan.sub_worker]
+    q_cpu = wl.q.cpu().view(N, Hq, D)
+    eo_d, el_d, _ = O.forward_decode(dplan, q_cpu[:W], k_cpu, v_cpu, rope)
+    eo_p, el_p = O.forward_prefill_batch(pplan, q_cpu[W:], k_cpu, v_cpu, rope)
+    assert_close(out[:W], eo_d, op.dtype, "decode rows")
+    assert_close(lse[:W], el_d, op.dtype, "decode lse")
+    assert_close(out[W:], eo_p, op.dtype, "prefill rows")
+    assert_close(lse[W:], el_p, op.dtype, "prefill lse")
