@@ -136,6 +136,20 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
+// Workgroup -> (work item, kv head).  The hardware hands workgroup b of a launch to die b % 8
+// (8 dies, one L2 each).  The planner lays the items out so that item i belongs on die i % 8;
+// here the kv heads of an item are placed at consecutive turns of that same die, so the
+// workgroups that read the same tokens (one per head: adjacent 2*D-byte pieces of each pool
+// row) run on one die at the same time.  n_items is a multiple of 8.
+struct ItemHead {
+  int item, head;
+};
+__device__ __forceinline__ ItemHead item_and_head(unsigned b, int num_kv_heads) {
+  const unsigned die = b & 7u, turn = b >> 3;
+  const unsigned head = turn % (unsigned)num_kv_heads, slot = turn / (unsigned)num_kv_heads;
+  return ItemHead{(int)(slot * 8u + die), (int)head};
+}
+
 // physical slot of token t of a sub-request
 __device__ __forceinline__ long long kv_slot(const int32_t* kv_indices, int kv_begin, int t, int page_size,
                                              bool slots) {

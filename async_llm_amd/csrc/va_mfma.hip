@@ -56,8 +56,25 @@ constexpr int kTileTokens = 32;
 #define VA_MFMA_MIN_BLOCKS 2  // workgroups per CU the register allocation must allow
 #endif
 
+#if VA_NARROW_EXPERIMENT == 2  // per-workgroup timeline: start, prologue end, loop end, end, hardware id
+__device__ unsigned long long va_debug_times[5 * 16384];
+extern "C" __attribute__((visibility("default"))) int va_debug_read(void* host, size_t bytes) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(va_debug_times), bytes);
+}
+#define VA_STAMP(k) \
+  if (threadIdx.x == 0 && blockIdx.x < 16384) va_debug_times[5 * blockIdx.x + (k)] = wall_clock64();
+#else
+#define VA_STAMP(k)
+#endif
+
 template <typename E, int kD>
 __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_kernel(AttnArgs a) {
+  VA_STAMP(0)
+#if VA_NARROW_EXPERIMENT == 2
+  if (threadIdx.x == 0 && blockIdx.x < 16384)
+    va_debug_times[5 * blockIdx.x + 4] = __builtin_amdgcn_s_getreg(4 | (31 << 11)) |
+                                         ((unsigned long long)__builtin_amdgcn_s_getreg(20 | (31 << 11)) << 32);
+#endif
   using S = typename E::storage;
   constexpr int kSteps = kD / 32;     // contraction steps of Q.K^T
   constexpr int kDimTiles = kD / 16;  // 16-dim tiles of the output
@@ -69,10 +86,12 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
   __shared__ float o_s[2][16][kD + 4];
   __shared__ float ml_s[2][16][2];
 
-  const int32_t* item = a.items + (long long)blockIdx.x * VA_ITEM_WORDS;
-  const int hk = blockIdx.y;
+  const ItemHead where = item_and_head(blockIdx.x, a.num_kv_heads);
+  const int32_t* item = a.items + (long long)where.item * VA_ITEM_WORDS;
+  const int hk = where.head;
   const int G = a.num_q_heads / a.num_kv_heads;
   const int n_q = item[VA_I_N_Q];
+  if (n_q == 0) return;  // padding item: keeps the launch order aligned with the die round-robin
   const int part_base = item[VA_I_PART_BASE];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -166,6 +185,7 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
       }
     };
 
+    VA_STAMP(1)
     int t0 = link[VA_L_TOK_BEGIN] + wave * kTileTokens;
     if (t0 < t_stop) {
       va_u32x4 kf[2][kSteps];
@@ -241,6 +261,7 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
     }
   }
 
+  VA_STAMP(2)
   // row sums live spread over the four contraction groups
   l_run += __shfl_xor(l_run, 16, kWave);
   l_run += __shfl_xor(l_run, 32, kWave);
@@ -306,12 +327,13 @@ __global__ __launch_bounds__(kMfmaThreads, VA_MFMA_MIN_BLOCKS) void attn_mfma_ke
       }
     }
   }
+  VA_STAMP(3)
 }
 
 template <typename E>
 static int launch_mfma_typed(const AttnArgs& a, int n_items, hipStream_t stream) {
   if (n_items == 0) return VA_OK;
-  const dim3 grid((unsigned)n_items, (unsigned)a.num_kv_heads), block(kMfmaThreads);
+  const dim3 grid((unsigned)n_items * (unsigned)a.num_kv_heads), block(kMfmaThreads);
   switch (a.head_dim) {
     case 64:
       hipLaunchKernelGGL((attn_mfma_kernel<E, 64>), grid, block, 0, stream, a);

@@ -51,10 +51,12 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   auto k_tile = [&](int b) __attribute__((always_inline)) { return smem + (b * 2) * kWideTokens * kRow; };
   auto v_tile = [&](int b) __attribute__((always_inline)) { return smem + (b * 2 + 1) * kWideTokens * kRow; };
 
-  const int32_t* item = a.items + (long long)blockIdx.x * VA_ITEM_WORDS;
-  const int hk = blockIdx.y;
+  const ItemHead where = item_and_head(blockIdx.x, a.num_kv_heads);
+  const int32_t* item = a.items + (long long)where.item * VA_ITEM_WORDS;
+  const int hk = where.head;
   const int G = a.num_q_heads / a.num_kv_heads;
   const int n_q = item[VA_I_N_Q];
+  if (n_q == 0) return;  // padding item: keeps the launch order aligned with the die round-robin
   const int part_base = item[VA_I_PART_BASE];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -335,7 +337,7 @@ static int launch_wide_one(const AttnArgs& a, int n_items, hipStream_t stream) {
     if (e != hipSuccess) return va_fail(VA_ERR_HIP, "raising the LDS limit: %s", hipGetErrorString(e));
     configured = true;
   }
-  const dim3 grid((unsigned)n_items, (unsigned)a.num_kv_heads), block(kWideThreads);
+  const dim3 grid((unsigned)n_items * (unsigned)a.num_kv_heads), block(kWideThreads);
   hipLaunchKernelGGL((attn_mfma_wide_kernel<E, kD>), grid, block, bytes, stream, a);
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? VA_OK : va_fail(VA_ERR_HIP, "wide attention launch: %s", hipGetErrorString(e));

@@ -30,7 +30,9 @@ namespace {
 
 struct Item {
   int32_t link_begin, n_links, n_q, part_base, tokens, kind;
+  int32_t unit;  // items that stream the same K/V chunk share a unit (planner only, not serialised)
 };
+constexpr int kXcds = 8;  // accelerator dies of an MI355X, each with its own L2; workgroup b runs on die b % 8
 struct Link {
   int32_t kv_begin, tok_begin, tok_end, qref, causal_base, flags;
 };
@@ -239,10 +241,12 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   };
   std::vector<Pending> pend;
 
-  auto emit = [&](int32_t n_q, const std::vector<Link>& links, std::vector<int32_t>&& rows) {
+  int32_t next_unit = 0;
+  auto emit = [&](int32_t n_q, const std::vector<Link>& links, std::vector<int32_t>&& rows, int32_t unit = -1) {
     int32_t tokens = 0;
     for (auto& l : links) tokens += l.tok_end - l.tok_begin;
-    Item it{(int32_t)out.links.size(), (int32_t)links.size(), n_q, -1, tokens, n_q > q_tile ? 1 : 0};
+    Item it{(int32_t)out.links.size(), (int32_t)links.size(), n_q, -1, tokens, n_q > q_tile ? 1 : 0,
+            unit >= 0 ? unit : next_unit++};
     out.links.insert(out.links.end(), links.begin(), links.end());
     for (int32_t r : rows) ++row_count[r];
     pend.push_back(Pending{(int32_t)out.items.size(), std::move(rows)});
@@ -271,11 +275,11 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
       tile_qref.push_back((int32_t)out.qrefs.size());
       out.qrefs.insert(out.qrefs.end(), gr.subrows.begin() + tl.first, gr.subrows.begin() + tl.second);
     }
-    auto emit_range = [&](size_t ti, int32_t t0, int32_t t1) {
+    auto emit_range = [&](size_t ti, int32_t t0, int32_t t1, int32_t unit = -1) {
       const size_t a = tiles[ti].first, b = tiles[ti].second;
       std::vector<int32_t> rows;
       for (size_t r = a; r < b; ++r) rows.push_back((int32_t)s->sub_worker[gr.subrows[r]]);
-      emit((int32_t)(b - a), {Link{s->kv_indptr[rep], t0, t1, tile_qref[ti], VA_NO_CAUSAL, lflags}}, std::move(rows));
+      emit((int32_t)(b - a), {Link{s->kv_indptr[rep], t0, t1, tile_qref[ti], VA_NO_CAUSAL, lflags}}, std::move(rows), unit);
     };
     auto chunk_len = [&](int32_t chunk) {
       const int32_t n_chunks = (len + chunk - 1) / chunk;
@@ -283,9 +287,11 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     };
     // narrow tiles: chunk-major; wide tiles: their own (finer) chunking
     const int32_t per = chunk_len(kv_chunk);
-    for (int32_t t0 = 0; t0 < len; t0 += per)
+    for (int32_t t0 = 0; t0 < len; t0 += per) {
+      const int32_t unit = next_unit++;  // the narrow tiles of one chunk: same die, side by side
       for (size_t ti = 0; ti < tiles.size(); ++ti)
-        if (tiles[ti].second - tiles[ti].first <= q_tile) emit_range(ti, t0, std::min(len, t0 + per));
+        if (tiles[ti].second - tiles[ti].first <= q_tile) emit_range(ti, t0, std::min(len, t0 + per), unit);
+    }
     const int32_t per_w = chunk_len(wide_chunk);
     for (size_t ti = 0; ti < tiles.size(); ++ti)
       if (tiles[ti].second - tiles[ti].first > q_tile)
@@ -372,20 +378,78 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     else if (parts_of_row[r].empty()) out.row_flags[r] = VA_ROW_DIRECT;
   }
 
-  // wide items first, then narrow ones; within a class longest first, so the tail of each
-  // launch is made of short items
-  std::vector<int32_t> order(out.items.size());
-  std::iota(order.begin(), order.end(), 0);
-  std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) {
-    const Item &ix = out.items[x], &iy = out.items[y];
-    if (ix.kind != iy.kind) return ix.kind > iy.kind;
-    return (int64_t)ix.tokens * ix.n_q > (int64_t)iy.tokens * iy.n_q;
-  });
+  // Launch order.  Wide items first (their own launch), then narrow ones.  The hardware hands
+  // workgroup b of a launch to die b % 8, and each die has its own L2, so within a class:
+  //   * units (the tiles that stream one K/V chunk) are dealt to the 8 dies, heaviest first, each
+  //     to the least loaded die, and stay together there: the chunk is fetched from HBM by one
+  //     tile and found in that die's L2 by the others;
+  //   * after a first round of mixed sizes a die runs its units longest item first, so the tail of
+  //     the launch is made of short items;
+  //   * position p of the class holds entry p / 8 of die p % 8; dies with fewer entries are
+  //     padded with empty items (n_q = 0, the kernels return at once), which also keeps the
+  //     class a multiple of 8 long so the next kv head starts on die 0 again.
   std::vector<Item> sorted;
-  sorted.reserve(order.size());
-  for (int32_t i : order) {
-    sorted.push_back(out.items[i]);
-    out.n_wide += out.items[i].kind;
+  sorted.reserve(out.items.size() + 2 * kXcds);
+  for (int kind = 1; kind >= 0; --kind) {
+    struct Unit {
+      int64_t cost = 0, item_cost = 0;
+      std::vector<int32_t> members;
+    };
+    std::vector<Unit> units;
+    std::unordered_map<int32_t, int32_t> unit_index;
+    for (int32_t i = 0; i < (int32_t)out.items.size(); ++i) {
+      const Item& it = out.items[i];
+      if (it.kind != kind) continue;
+      auto at = unit_index.find(it.unit);
+      if (at == unit_index.end()) {
+        at = unit_index.emplace(it.unit, (int32_t)units.size()).first;
+        units.emplace_back();
+      }
+      Unit& u = units[at->second];
+      const int64_t cost = it.tokens;  // a tile streams its tokens once whatever its row count
+      u.cost += cost;
+      u.item_cost = std::max(u.item_cost, cost);
+      u.members.push_back(i);
+    }
+    if (units.empty()) continue;
+    std::vector<int32_t> by_cost(units.size());
+    std::iota(by_cost.begin(), by_cost.end(), 0);
+    std::stable_sort(by_cost.begin(), by_cost.end(), [&](int32_t x, int32_t y) { return units[x].cost > units[y].cost; });
+    int64_t load[kXcds] = {0};
+    std::vector<int32_t> die_units[kXcds];
+    for (int32_t u : by_cost) {
+      const int die = (int)(std::min_element(load, load + kXcds) - load);
+      die_units[die].push_back(u);
+      load[die] += units[u].cost;
+    }
+    std::vector<int32_t> die_items[kXcds];
+    size_t depth = 0;
+    for (int d = 0; d < kXcds; ++d) {
+      std::stable_sort(die_units[d].begin(), die_units[d].end(),
+                       [&](int32_t x, int32_t y) { return units[x].item_cost > units[y].item_cost; });
+      // Workgroups that start together and stream the same number of tokens also finish together,
+      // and while they all write results and set up their next item the memory system idles.  So
+      // the first round of a die (the items that start at once: 64 workgroup slots) is a spread
+      // sample of all its sizes; their staggered ends keep the later rounds out of step.
+      const size_t n_u = die_units[d].size();
+      const size_t first_round = std::min<size_t>(n_u, std::max(1, 64 / shape->num_kv_heads));
+      if (first_round > 1 && n_u > first_round) {
+        std::vector<int32_t> head, rest;
+        std::vector<char> picked(n_u, 0);
+        for (size_t k = 0; k < first_round; ++k) picked[k * (n_u - 1) / (first_round - 1)] = 1;
+        for (size_t i = 0; i < n_u; ++i) (picked[i] ? head : rest).push_back(die_units[d][i]);
+        head.insert(head.end(), rest.begin(), rest.end());
+        die_units[d].swap(head);
+      }
+      for (int32_t u : die_units[d])
+        die_items[d].insert(die_items[d].end(), units[u].members.begin(), units[u].members.end());
+      depth = std::max(depth, die_items[d].size());
+    }
+    const Item padding{0, 0, 0, -1, 0, kind, -1};
+    for (size_t slot = 0; slot < depth; ++slot)
+      for (int d = 0; d < kXcds; ++d)
+        sorted.push_back(slot < die_items[d].size() ? out.items[die_items[d][slot]] : padding);
+    if (kind == 1) out.n_wide = (int32_t)sorted.size();
   }
   out.items.swap(sorted);
   return VA_OK;

@@ -154,10 +154,12 @@ __global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
   __shared__ float acc_s[kGenWaves][kHB][kD];
   __shared__ float ml_s[kGenWaves][kHB][2];
 
-  const int32_t* item = a.items + (long long)blockIdx.x * VA_ITEM_WORDS;
-  const int hk = blockIdx.y;
+  const ItemHead where = item_and_head(blockIdx.x, a.num_kv_heads);
+  const int32_t* item = a.items + (long long)where.item * VA_ITEM_WORDS;
+  const int hk = where.head;
   const int G = a.num_q_heads / a.num_kv_heads;
   const int n_q = item[VA_I_N_Q];
+  if (n_q == 0) return;  // padding item: keeps the launch order aligned with the die round-robin
   const int part_base = item[VA_I_PART_BASE];
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
@@ -380,7 +382,7 @@ __global__ __launch_bounds__(64) void merge_kernel(MergeArgs a) {
 
 template <typename E>
 int launch_generic(const AttnArgs& a, int n_items, hipStream_t stream) {
-  const dim3 grid((unsigned)n_items, (unsigned)a.num_kv_heads), block(kGenThreads);
+  const dim3 grid((unsigned)n_items * (unsigned)a.num_kv_heads), block(kGenThreads);
   constexpr int kMaxD = 16 / sizeof(typename E::storage) * 64;
   switch (a.head_dim) {
 #define VA_CASE(D)                                                              \
@@ -470,6 +472,10 @@ extern "C" int va_attention(const void* q_dev, int64_t q_row_stride, const void*
   if (h[VA_H_MAGIC] != VA_PLAN_MAGIC) return va_fail(VA_ERR_ARG, "plan header has no magic word");
   const int n_rows = h[VA_H_N_ROWS], n_items = h[VA_H_N_ITEMS], n_partials = h[VA_H_N_PARTIALS];
   if (n_rows == 0) return VA_OK;
+  // the kernels map workgroup -> (item, head) assuming each launch covers a multiple of 8 items
+  if (n_items % 8 || h[VA_H_N_WIDE] % 8 || h[VA_H_N_WIDE] < 0 || h[VA_H_N_WIDE] > n_items)
+    return va_fail(VA_ERR_ARG, "plan header: item counts (%d, %d wide) are not padded to the 8 dies", n_items,
+                   h[VA_H_N_WIDE]);
   if (!out_dev) return va_fail(VA_ERR_ARG, "null out");
   if (n_items > 0 && (!q_dev || !k_pool_dev || !v_pool_dev || !sub_worker_dev || !sub_loc_dev || !kv_indices_dev))
     return va_fail(VA_ERR_ARG, "null pointer");

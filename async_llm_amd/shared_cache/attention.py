@@ -167,7 +167,15 @@ class SharedCacheAttention:
         if kernel == "auto" and self.rotary_dim % 16:
             kernel = "generic"  # the matrix-core kernel rotates queries in 8-element pieces
         self.kernel = kernel
-        self.plan_params = native.VaPlanParams(_KERNELS[kernel], 0, 0, 0, 0)
+        # planner knobs (0 = let the planner choose); VIEWATTN_PLAN="kv_chunk=1024,target_items=768" overrides
+        knobs = dict(q_tile=0, kv_chunk=0, target_items=0, wide_tile=0)
+        for part in filter(None, os.environ.get("VIEWATTN_PLAN", "").split(",")):
+            name, _, value = part.partition("=")
+            if name.strip() not in knobs:
+                raise ValueError(f"VIEWATTN_PLAN: unknown knob {name!r} (known: {sorted(knobs)})")
+            knobs[name.strip()] = int(value)
+        self.plan_params = native.VaPlanParams(_KERNELS[kernel], knobs["q_tile"], knobs["kv_chunk"],
+                                               knobs["target_items"], knobs["wide_tile"])
         self._shape = native.make_shape(num_qo_heads, num_kv_heads, head_dim, page_size, dtype)
         self._rope_desc: Optional[native.VaRope] = None
         self._workspace: Optional[torch.Tensor] = None

@@ -74,8 +74,14 @@ def check_coverage(blob, qo, kvp, lens, flags, sub_worker, n_rows):
     seen = {}
     part_owner = {}
     contributions = [0] * n_rows
+    # each class (wide first, then narrow) is padded to a multiple of the 8 dies
+    assert h[H["N_WIDE"]] % 8 == 0 and h[H["N_ITEMS"]] % 8 == 0
+    assert all(it[5] == 1 for it in items[: h[H["N_WIDE"]]]) and all(it[5] == 0 for it in items[h[H["N_WIDE"]]:])
     for it in items:
         lb, nl, nq, part_base = it[0], it[1], it[2], it[3]
+        if nq == 0:  # padding item
+            assert nl == 0 and part_base == -1
+            continue
         assert nl >= 1 and 1 <= nq <= max(h[H["Q_TILE"]], h[H["WIDE_TILE"]])
         assert it[5] == int(nq > h[H["Q_TILE"]])  # kind: wide iff more rows than the narrow tile
         rows_of_item = None
@@ -216,8 +222,46 @@ def test_readers_of_one_block_share_a_tile():
     rc, blob, counts = build_plan(qo, kvp, kvi, lens, flags, chain, sw, 6, page=page, q_tile=4, kv_chunk=1024)
     assert rc == 0
     h, items, links, qrefs, *_ = decode_plan(blob)
-    assert sorted(int(i[2]) for i in items) == [2, 4]  # 6 readers -> tiles of 4 and 2 rows, one chunk each
+    assert sorted(int(i[2]) for i in items if i[2]) == [2, 4]  # 6 readers -> tiles of 4 and 2 rows, one chunk each
     check_coverage(blob, qo, kvp, lens, flags, sw, 6)
+
+
+def test_tiles_of_one_chunk_run_on_one_die():
+    """Workgroup b of a launch runs on die b % 8 (each die has its own L2): the tiles
+    that stream the same chunk of a shared block sit at consecutive slots of ONE die,
+    and the dies carry about the same load."""
+    page, L = 16, 2048
+    shared = list(range(L // page))
+    qo, kvp, kvi, lens, flags, chain, sw = [0], [0], [], [], [], [], []
+    n_req = 24
+    for w in range(n_req):  # every request reads the shared block ...
+        kvi += shared
+        kvp.append(len(kvi)); lens.append(L); flags.append(0); chain.append(-1); sw.append(w); qo.append(len(sw))
+    rng = random.Random(5)
+    for w in range(n_req):  # ... and a private one
+        n = rng.randint(100, 1500)
+        kvi += [1000 + 100 * w + i for i in range(-(-n // page))]
+        kvp.append(len(kvi)); lens.append(n); flags.append(0); chain.append(-1); sw.append(w); qo.append(len(sw))
+    rc, blob, counts = build_plan(qo, kvp, kvi, lens, flags, chain, sw, n_req, page=page, q_tile=4, kv_chunk=256)
+    assert rc == 0
+    h, items, links, *_ = decode_plan(blob)
+    assert h[H["N_WIDE"]] == 0
+    where = {}
+    load = [0] * 8
+    for pos, it in enumerate(items):
+        if it[2] == 0:
+            continue
+        l = links[it[0]]
+        load[pos % 8] += int(it[4])
+        if l[0] == 0:  # kv_begin of the shared block's representative
+            where.setdefault(int(l[1]), []).append(pos)
+    assert len(where) == L // 256 and all(len(v) == n_req // 4 for v in where.values())
+    for t0, positions in where.items():
+        assert len({p % 8 for p in positions}) == 1, (t0, positions)
+        slots = sorted(p // 8 for p in positions)
+        assert slots == list(range(slots[0], slots[0] + len(slots)))
+    assert max(load) <= 1.25 * (sum(load) / 8) + 256
+    check_coverage(blob, qo, kvp, lens, flags, sw, n_req)
 
 
 def test_plan_rejects_inconsistent_tables():
