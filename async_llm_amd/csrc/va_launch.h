@@ -46,5 +46,6 @@ struct MergeArgs {
 // `n_wide` leading items are wide tiles (va_mfma_wide.hip), the rest narrow ones.
 int launch_mfma(const AttnArgs& a, int dtype, int n_items, int n_wide, int q_tile, hipStream_t stream);
 int launch_mfma_wide(const AttnArgs& a, int dtype, int n_items, hipStream_t stream);
+int launch_mfma_stream(const AttnArgs& a, int dtype, int n_items, hipStream_t stream);
 
 }  // namespace va

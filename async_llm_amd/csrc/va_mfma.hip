@@ -366,7 +366,11 @@ int launch_mfma(const AttnArgs& a_in, int dtype, int n_items, int n_wide, int q_
   }
   a.items += (long long)n_wide * VA_ITEM_WORDS;
   const int n_narrow = n_items - n_wide;
+#if VA_NARROW_REGISTER_PATH  // the older register-staged kernel, kept for comparison builds
   return dtype == VA_BF16 ? launch_mfma_typed<BF16>(a, n_narrow, stream) : launch_mfma_typed<F16>(a, n_narrow, stream);
+#else
+  return launch_mfma_stream(a, dtype, n_narrow, stream);
+#endif
 }
 
 }  // namespace va

@@ -10,6 +10,9 @@ typedef float va_f32x4 __attribute__((ext_vector_type(4)));
 
 typedef float va_f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t va_u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes as a plain vector (registers, LDS)
+typedef uint32_t va_u32x2 __attribute__((ext_vector_type(2)));
+typedef short va_i16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 va_f16x4 __attribute__((ext_vector_type(4)));
 
 namespace va {
 
@@ -27,6 +30,11 @@ struct Mma<BF16> {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(va_bf16x8, a), __builtin_bit_cast(va_bf16x8, b),
                                                    c, 0, 0, 0);
   }
+  // 16x16x16: four contraction elements per lane
+  static __device__ __forceinline__ va_f32x4 run16(const va_u32x2& a, const va_u32x2& b, va_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(va_i16x4, a), __builtin_bit_cast(va_i16x4, b),
+                                                     c, 0, 0, 0);
+  }
   static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
     const __bf16 l = (__bf16)lo, h = (__bf16)hi;
     return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
@@ -43,6 +51,10 @@ struct Mma<F16> {
   static __device__ __forceinline__ va_f32x4 run(const A& a, const B& b, va_f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(va_f16x8, a), __builtin_bit_cast(va_f16x8, b), c,
                                                   0, 0, 0);
+  }
+  static __device__ __forceinline__ va_f32x4 run16(const va_u32x2& a, const va_u32x2& b, va_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(va_f16x4, a), __builtin_bit_cast(va_f16x4, b), c,
+                                                 0, 0, 0);
   }
   static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
     const _Float16 l = (_Float16)lo, h = (_Float16)hi;
