@@ -35,6 +35,13 @@ constexpr int kStreamThreads = 256;
 constexpr int kStreamWaves = 4;
 constexpr int kStreamTok = 16;  // tokens per tile
 
+#ifndef VA_STREAM_BUFFERS_256
+#define VA_STREAM_BUFFERS_256 3
+#endif
+#ifndef VA_STREAM_BLOCKS_256
+#define VA_STREAM_BLOCKS_256 3
+#endif
+
 template <int kD>
 struct StreamShape {
   static constexpr int kChunks = kD / 8;                     // 16-byte pieces of a head row
@@ -43,8 +50,8 @@ struct StreamShape {
   static constexpr int kLoadsPerKind = kStreamTok / kRowsPerLoad;  // loads per K (or V) tile
   static constexpr int kLoadsPerWave = 2 * kLoadsPerKind / kStreamWaves;
   static constexpr int kTileUnits = kStreamTok * kChunks;    // 16-byte units of a K (or V) tile
-  static constexpr int kBuffers = kD == 256 ? 3 : 4;         // ring depth: 48 KB at D=256, 32 KB, 16 KB
-  static constexpr int kMinBlocks = kD == 256 ? 3 : 4;       // workgroups per CU (registers and LDS allow)
+  static constexpr int kBuffers = kD == 256 ? VA_STREAM_BUFFERS_256 : 4;         // ring depth: 48 KB at D=256, 32 KB, 16 KB
+  static constexpr int kMinBlocks = kD == 256 ? VA_STREAM_BLOCKS_256 : 4;       // workgroups per CU (registers and LDS allow)
   static constexpr int kPvWaves = kD >= 128 ? 4 : 2;         // waves that own a slice of the head dim
   static constexpr int kDimsPerWave = kD / kPvWaves;
   static constexpr int kRun = kDimsPerWave / 16;             // contiguous dims a lane reads per V token
@@ -159,16 +166,18 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
 
     // Request tile i (tokens tok_begin + 16 i ..) into ring buffer i % kBuffers.  Rows past the
     // visible range re-read the last visible token (their scores are masked).
-    auto issue = [&](int i, auto uniform_tag) __attribute__((always_inline)) {
+    // page of tile i (uniform page tables).  Read through the constant address space: the table is
+    // read-only for the kernel, and this keeps the lookup a scalar load (a vector load would have
+    // to be waited for together with every tile load in flight).
+    auto page_of = [&](int i) __attribute__((always_inline)) {
+      return ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + (tok_begin + i * kStreamTok) / P];
+    };
+    auto issue = [&](int i, auto uniform_tag, int page) __attribute__((always_inline)) {
       constexpr bool kUniform = decltype(uniform_tag)::value;
       const int t0 = tok_begin + i * kStreamTok;
       va_u32x4* buf = ring + (i % kBuffers) * 2 * kTileUnits;
       long long base_byte = 0;  // wave-uniform: pool byte offset of the tile's first token
       if constexpr (kUniform) {
-        // read through the constant address space: the table is read-only for the kernel, and this
-        // keeps the lookup a scalar load (a vector load would have to be waited for together with
-        // every tile load in flight)
-        const int page = ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + t0 / P];
         base_byte = ((long long)page * P + t0 % P) * row_bytes;
       }
       const int last_row = t_last - t0;  // rows beyond it are clamped
@@ -195,7 +204,7 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     auto first_tiles = [&](auto uniform_tag) __attribute__((always_inline)) {
 #pragma unroll
       for (int i = 0; i < kBuffers - 1; ++i)
-        if (i < n_tiles) issue(i, uniform_tag);
+        if (i < n_tiles) issue(i, uniform_tag, decltype(uniform_tag)::value ? page_of(i) : 0);
     };
     if (uniform_pages) {
       first_tiles(std::true_type{});
@@ -227,7 +236,7 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
 
     // ---- the tile loop, once per page-table kind so neither carries the other's branches ----
     auto stream = [&](auto uniform_tag) __attribute__((always_inline)) {
-    if (kBuffers - 1 < n_tiles) issue(kBuffers - 1, uniform_tag);
+    if (kBuffers - 1 < n_tiles) issue(kBuffers - 1, uniform_tag, decltype(uniform_tag)::value ? page_of(kBuffers - 1) : 0);
     for (int i = 0; i < n_tiles; ++i) {
       // This wave's loads of tile i have landed once at most the loads of the tiles requested
       // after it are outstanding; the barrier then covers the other waves' loads.
@@ -237,6 +246,10 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
         ring_barrier<0>();
       }
 
+      // the page of the tile requested at the end of this iteration: looked up now, so the lookup's
+      // latency is covered by the computation
+      const bool refill = i + kBuffers < n_tiles;
+      const int next_page = (decltype(uniform_tag)::value && refill) ? page_of(i + kBuffers) : 0;
       const int t0 = tok_begin + i * kStreamTok;
       const char* kt = lds + (i % kBuffers) * kBufferBytes;
       const char* vt = kt + kTileUnits * 16;
@@ -294,9 +307,9 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
         }
       }
       // refill this tile's buffer once every wave has consumed it
-      if (i + kBuffers < n_tiles) {
+      if (refill) {
         ring_barrier<kAnyInFlight>();
-        issue(i + kBuffers, uniform_tag);
+        issue(i + kBuffers, uniform_tag, next_page);
       }
     }
     };

@@ -122,7 +122,8 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     constexpr int kTokStep = kWideThreads / kChunks;  // tokens per round of loads
     constexpr int kRounds = kWideTokens / kTokStep;
     const int ld_tok = tid / kChunks, ld_c = tid - ld_tok * kChunks;
-    const bool uniform_pages = !slots && (P % 16 == 0);
+    // a 16-token half tile lies inside one page only if the link starts on a 16-token boundary
+    const bool uniform_pages = !slots && (P % 16 == 0) && (tok_begin % 16 == 0);
     va_u32x4 stage_k[kRounds], stage_v[kRounds];
     auto fetch = [&](int t0) __attribute__((always_inline)) {
       if (uniform_pages) {
