@@ -42,8 +42,8 @@ struct MergeArgs {
   int num_q_heads, head_dim;
 };
 
-// Matrix-core attention (va_mfma.hip).
-// `n_wide` leading items are wide tiles (va_mfma_wide.hip), the rest narrow ones.
+// Matrix-core attention (launched from va_mfma.hip).
+// `n_wide` leading items are wide tiles (va_mfma_wide.hip), the rest narrow ones (va_mfma_stream.hip).
 int launch_mfma(const AttnArgs& a, int dtype, int n_items, int n_wide, int q_tile, hipStream_t stream);
 int launch_mfma_wide(const AttnArgs& a, int dtype, int n_items, hipStream_t stream);
 int launch_mfma_stream(const AttnArgs& a, int dtype, int n_items, hipStream_t stream);

@@ -44,7 +44,7 @@ enum {
   VA_I_N_Q,        // query rows in the tile
   VA_I_PART_BASE,  // first partial slot (one per query row), or -1: write `out` directly
   VA_I_TOKENS,     // KV tokens the item walks (scheduling weight)
-  VA_I_KIND,       // 1: wide tile (more rows than the narrow kernel's tile)
+  VA_I_KIND,       // 1: wide tile (more rows than the streaming kernel's tile)
 };
 
 // link word indices

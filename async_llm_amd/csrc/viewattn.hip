@@ -1,5 +1,5 @@
 // libviewattn.so: C ABI, rotation/store kernel, vector-ALU attention kernel and
-// the partial-state merge kernel.  The matrix-core kernels live in va_mfma.hip.
+// the partial-state merge kernel.  The matrix-core kernels live in va_mfma_stream.hip and va_mfma_wide.hip.
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>

@@ -32,6 +32,16 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
+# HBM bytes one launch (attention + merge) moves at the default sizes, from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs of this script scaled by the readings of --workload
+# copy_calibration (bytes = 2 KiB x FETCH_SIZE + 1 KiB x WRITE_SIZE); the summaries are in
+# profiles/.  A counter run cannot be made from inside the timed process, so the figure is
+# carried here and only reported for the configuration it was measured on.
+MEASURED_TRAFFIC_BYTES = {
+    ("batched_decode", "mfma"): (2_341_550 + 15_020 + 14_840 + 512) * 1024,
+    ("view_prefill", "mfma"): (2 * 7_062_999 + 131_109) * 1024,
+}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -39,7 +49,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=40)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="batched_decode",
-                    choices=["batched_decode", "mrope_decode", "view_prefill", "plumbing_decode", "mixed_batch"])
+                    choices=["batched_decode", "mrope_decode", "view_prefill", "plumbing_decode", "mixed_batch",
+                             "copy_calibration"])
     ap.add_argument("--layers", type=int, default=4, help="copies of the KV pool rotated over")
     ap.add_argument("--kernel", default=None, choices=[None, "auto", "generic", "mfma"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -147,6 +158,26 @@ def cpu_baseline(wl, sample):
     return t, sample_bytes, cores, what, n
 
 
+def copy_calibration(dev, steps):
+    """A plain device copy of known size (1 GiB read + 1 GiB written per launch):
+    what the FETCH_SIZE / WRITE_SIZE counters read for it gives the factor that
+    turns their readings for the attention kernels into bytes."""
+    import torch
+
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(3)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    print(json.dumps({"workload": "copy_calibration", "bytes_read": n, "bytes_written": n, "steps": steps,
+                      "ms_per_copy": round(ms, 4), "gbps_read_plus_write": round(2 * n / ms / 1e6, 1)}), flush=True)
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -160,6 +191,8 @@ def main() -> int:
         return 2
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "copy_calibration":
+        return copy_calibration(dev, args.steps)
     wl = build_workload(args.workload, dev, args.layers, args.kernel)
     layers = args.layers
 
@@ -188,6 +221,8 @@ def main() -> int:
         achieved = wl.alg_flops / (kern_avg_ms * 1e-3) / 1e12
         roof = dict(bound="mfma", achieved=round(achieved, 2), peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
                     frac=round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), traffic=None)
+    if args.layers == 4 and not os.environ.get("VIEWATTN_PLAN"):
+        roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((wl.name, {1: "generic", 2: "mfma"}.get(counts.kernel)))
     roof.update(kernel="attention launch (all work items) + merge", kernel_ms_avg=round(kern_avg_ms, 4),
                 kernel_ms_median=round(kern_med_ms, 4))
 
@@ -206,7 +241,7 @@ def main() -> int:
         "roofline": roof,
     }
     if not args.no_cpu_baseline:
-        sample = args.cpu_sample or (8 if decode else 1)
+        sample = args.cpu_sample or (64 if decode else 2)
         t_cpu, sample_bytes, cores, what, n = cpu_baseline(wl, sample)
         if decode:
             cpu_value, cpu_unit = sample_bytes / t_cpu / 1e9, "GB/s"

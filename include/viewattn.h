@@ -147,7 +147,7 @@ typedef struct VaPlanCounts {
   int32_t kernel;        /* resolved kernel family */
   int32_t q_tile;        /* resolved */
   int32_t kv_chunk;      /* resolved */
-  int32_t n_items;
+  int32_t n_items;       /* work items incl. padding (multiple of 8) */
   int32_t n_links;
   int32_t n_qrefs;
   int32_t n_partials;    /* partial (row, item) slots the launch will write */
@@ -168,6 +168,10 @@ VA_API int va_plan_count(const VaSubRequests* subs, const VaShape* shape, const 
  * device verbatim and pass the device copy to va_attention.  Layout (int32
  * words): header[24] | items[n_items*8] | links[n_links*8] | qrefs[n_qrefs] |
  * row_part_indptr[n_rows+1] | row_part_ids[n_row_parts] | row_flags[n_rows].
+ * Items are in launch order, laid out for the 8 dies of an MI355X (workgroup b
+ * of a launch runs on die b % 8): wide items first, then narrow ones, each
+ * class padded with empty items (n_q = 0) to a multiple of 8; n_items and
+ * n_wide_items count the padding.
  */
 VA_API int va_plan_build(const VaSubRequests* subs, const VaShape* shape, const VaPlanParams* params,
                   int32_t* plan_host, int64_t plan_capacity_words, VaPlanCounts* counts);
