@@ -11,7 +11,7 @@ int va_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3))
 bool va_mfma_supported(int dtype, int head_dim, int gqa);
 int va_mfma_max_q_tile(int gqa);
 int va_mfma_default_q_tile(int gqa, bool has_chain);
-int va_mfma_wide_q_tile(int gqa);  // query rows of a wide tile (0: no wide kernel for this group size)
+int va_mfma_wide_q_tile(int gqa, int head_dim);  // query rows of a wide tile
 
 // Scratch for `n_partials` partial softmax states: fp32 accumulator rows plus
 // (max, sum) pairs, per q head.

@@ -22,7 +22,7 @@ int va_mfma_default_q_tile(int gqa, bool has_chain) {
   (void)has_chain;
   return 16 / gqa;
 }
-int va_mfma_wide_q_tile(int gqa) { return 128 / gqa; }
+int va_mfma_wide_q_tile(int gqa, int head_dim) { return (head_dim == 256 ? 128 : 256) / gqa; }
 
 namespace va {
 

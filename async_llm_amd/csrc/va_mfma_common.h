@@ -25,6 +25,15 @@ struct Mma<BF16> {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(va_bf16x8, a), __builtin_bit_cast(va_bf16x8, b),
                                                    c, 0, 0, 0);
   }
+  // Same product with the accumulator pinned in the accumulation registers (AGPRs).  Written as
+  // assembly because the register allocator otherwise treats AGPRs as spill space for a long-lived
+  // accumulator and copies all of it to VGPRs and back around every tile.  The leading s_nop covers
+  // the wait states between the vector ALU writing an operand and the matrix pipe reading it, which
+  // the compiler cannot insert for code it does not see; callers wait (accumulator_fence) before
+  // reading the accumulator with anything but another product.
+  static __device__ __forceinline__ void run32_acc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
   template <typename A, typename B>
   static __device__ __forceinline__ va_f32x4 run(const A& a, const B& b, va_f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(va_bf16x8, a), __builtin_bit_cast(va_bf16x8, b),
@@ -46,6 +55,9 @@ struct Mma<F16> {
   static __device__ __forceinline__ va_f32x16 run32(const A& a, const B& b, va_f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(va_f16x8, a), __builtin_bit_cast(va_f16x8, b), c,
                                                   0, 0, 0);
+  }
+  static __device__ __forceinline__ void run32_acc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
   template <typename A, typename B>
   static __device__ __forceinline__ va_f32x4 run(const A& a, const B& b, va_f32x4 c) {
@@ -91,6 +103,34 @@ __device__ __forceinline__ uint4 rotated_query_piece(const RopeDev& rope, const 
     out[w] = Mma<E>::pack(y[0], y[1]);  // y is already representable: the conversion is exact
   }
   return make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+// Wait until the matrix pipe has written the results of products issued from assembly
+// (run32_acc): 8 passes plus the write-back, 20 wait states.
+__device__ __forceinline__ void accumulator_fence() { asm volatile("s_nop 15\n\ts_nop 3" ::: "memory"); }
+
+// Workgroup barrier for the tile ring.  __syncthreads() carries a fence that waits for ALL
+// outstanding memory operations, which would drain the loads of the tiles still in flight; this
+// one waits until at most `n` of the wave's vector memory operations (the pool -> LDS loads) are
+// outstanding, and for the wave's own LDS traffic, before it joins the barrier.  The "memory"
+// clobber keeps the compiler from moving LDS accesses or loads across it.
+template <int n>
+__device__ __forceinline__ void ring_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(n) : "memory");
+}
+constexpr int kAnyInFlight = 63;  // vmcnt(63): no wait on vector memory at all
+
+// One wave-level pool -> LDS load: lane l's 16 bytes at `src` land at LDS byte address
+// `lds_base + 16 l` (lds_base is wave-uniform and travels in M0).  Written as assembly on purpose:
+// when the compiler sees such a load it makes every later LDS read wait for ALL of them
+// (it cannot tell the ring's buffers apart), which would serialise the ring.  Completion is
+// tracked by hand instead, with the vmcnt values of ring_barrier.
+__device__ __forceinline__ void load_to_lds(const void* src, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base)
+               : "memory");  // M0 is scratch for the compiler too: it sets it right before each use of its own
+}
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }
 
 }  // namespace va

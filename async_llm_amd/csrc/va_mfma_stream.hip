@@ -66,30 +66,6 @@ __device__ __forceinline__ int swz(int r) {
   return (r >> 1) & 7;
 }
 
-// Workgroup barrier for the tile ring.  __syncthreads() carries a fence that waits for ALL
-// outstanding memory operations, which would drain the loads of the tiles still in flight; this
-// one waits until at most `n` of the wave's vector memory operations (the pool -> LDS loads) are
-// outstanding, and for the wave's own LDS traffic, before it joins the barrier.  The "memory"
-// clobber keeps the compiler from moving LDS accesses or loads across it.
-template <int n>
-__device__ __forceinline__ void ring_barrier() {
-  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(n) : "memory");
-}
-constexpr int kAnyInFlight = 63;  // vmcnt(63): no wait on vector memory at all
-
-// One wave-level pool -> LDS load: lane l's 16 bytes at `src` land at LDS byte address
-// `lds_base + 16 l` (lds_base is wave-uniform and travels in M0).  Written as assembly on purpose:
-// when the compiler sees such a load it makes every later LDS read wait for ALL of them
-// (it cannot tell the ring's buffers apart), which would serialise the ring.  Completion is
-// tracked by hand instead, with the vmcnt values of ring_barrier.
-__device__ __forceinline__ void load_to_lds(const void* src, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base)
-               : "memory");  // M0 is scratch for the compiler too: it sets it right before each use of its own
-}
-__device__ __forceinline__ uint32_t lds_address(const void* p) {
-  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
-}
-
 template <typename E, int kD>
 __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void attn_stream_kernel(AttnArgs a) {
   using S = typename E::storage;
@@ -116,6 +92,8 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
   const S* kp = (const S*)a.k_pool + (long long)hk * kD;
   const S* vp = (const S*)a.v_pool + (long long)hk * kD;
   const int P = a.page_size;
+  const bool pow2_pages = (P & (P - 1)) == 0;
+  const int p_shift = __builtin_ctz(P);  // t / P and t % P as shift and mask (power-of-two pages)
 
   // This lane's part of wave-level load u of a tile: tile row, and byte offset of the piece it
   // fetches within the head row (the piece that belongs at the lane's LDS position).
@@ -157,7 +135,7 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     const int causal_base = link[VA_L_CAUSAL_BASE];
     const bool slots = lflags & VA_LINK_SLOTS;
     // a 16-token tile lies inside one page: one wave-uniform page read per tile
-    const bool uniform_pages = !slots && (P % 16 == 0) && (tok_begin % 16 == 0);
+    const bool uniform_pages = !slots && pow2_pages && P >= 16 && (tok_begin % 16 == 0);
 
     const int t_stop = min(tok_end, causal_base + n_q);        // tokens any row of the tile sees
     const int t_row = min(tok_end, causal_base + row_iq + 1);  // tokens this lane's row sees
@@ -170,7 +148,7 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     // read-only for the kernel, and this keeps the lookup a scalar load (a vector load would have
     // to be waited for together with every tile load in flight).
     auto page_of = [&](int i) __attribute__((always_inline)) {
-      return ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + (tok_begin + i * kStreamTok) / P];
+      return ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + ((tok_begin + i * kStreamTok) >> p_shift)];
     };
     auto issue = [&](int i, auto uniform_tag, int page) __attribute__((always_inline)) {
       constexpr bool kUniform = decltype(uniform_tag)::value;
@@ -178,7 +156,7 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
       va_u32x4* buf = ring + (i % kBuffers) * 2 * kTileUnits;
       long long base_byte = 0;  // wave-uniform: pool byte offset of the tile's first token
       if constexpr (kUniform) {
-        base_byte = ((long long)page * P + t0 % P) * row_bytes;
+        base_byte = (((long long)page << p_shift) + (t0 & (P - 1))) * row_bytes;
       }
       const int last_row = t_last - t0;  // rows beyond it are clamped
 #pragma unroll

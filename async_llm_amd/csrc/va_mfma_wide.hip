@@ -1,24 +1,28 @@
-// Wide matrix-core view attention: query tiles of up to 128 MFMA rows.
+// Wide matrix-core view attention: query tiles of 128 (head_dim 256) or 256 MFMA rows, for
+// view-conditioned prefill (rows / G new tokens x G heads per workgroup).
 //
-// Used where many query rows meet the same keys: view-conditioned prefill
-// (128/G new tokens x G heads per workgroup) and decode over a block shared by
-// more than 16/G requests.  One workgroup of four waves per (work item, kv head);
-// wave w owns MFMA rows [32w, 32w+32) (row R = tile row R / G, head R % G) and
-// all four waves walk the same 32-token K/V tiles, which are staged once per
-// workgroup in LDS (double buffered: the global loads of tile i+1 are in flight
-// while tile i is computed, one barrier per tile).
+// One workgroup of four waves per (work item, kv head); wave w owns one or two blocks of 32
+// MFMA rows (row R = tile row R / G, head R % G).  All waves walk the same 32-token
+// K/V tiles, which travel pool -> LDS directly (global_load_lds_dwordx4) into a ring of four
+// buffers: three tiles are in flight while one is computed, one barrier per tile.
 //
-//   S^T[32 tokens, 32 rows] = K . Q^T     16 x v_mfma_f32_32x32x16 (D = 256), K from LDS as the A operand,
-//                                         the wave's rotated queries pinned in registers as B operands
+//   S^T[32 tokens, 32 rows] = K . Q^T    v_mfma_f32_32x32x16, K from LDS as the A operand; each K
+//                                        fragment is read once and used for all row blocks, whose
+//                                        rotated queries are pinned in registers as B operands
 //   online softmax per row (row = lane % 32; the other half-wave holds the other 16 tokens)
-//   O^T[D, 32 rows] += V^T . P^T          2 token steps x D/32 dim tiles; P is already laid out as the B operand
-//                                         (the token order of the contraction is chosen to match the S^T
-//                                         accumulator), V rows are read from LDS as 8 tokens x D/32 dims per
-//                                         lane and transposed in registers with v_perm_b32
+//   O^T[D, 32 rows] += V^T . P^T         2 token steps x D/32 dim tiles; P is already laid out as
+//                                        the B operand; V rows are read from LDS as 8 tokens x D/32
+//                                        dims per lane, transposed in registers with v_perm_b32, and
+//                                        each transposed fragment again serves all row blocks
 //
-// The query tile of the current link is rotated by all 256 threads into the (not yet
-// used) tile buffers, then each wave pulls its 32 rows into registers.
+// Two row blocks per wave halve the LDS bytes read per flop: with one block per wave the four
+// waves would need the whole LDS bandwidth of the CU just to feed the matrix pipe at its peak.
+// LDS rows are unpadded and swizzled (piece c of tile row r at position c ^ swz(r)), see
+// va_mfma_stream.hip.  The query tile is rotated by all 256 threads, one row block of every wave
+// (128 rows) at a time, into the two ring buffers that are not yet in use.
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "va_internal.h"
 #include "va_launch.h"
@@ -27,29 +31,54 @@
 namespace va {
 
 constexpr int kWideThreads = 256;
-constexpr int kWideRows = 128;   // MFMA rows per workgroup
+constexpr int kWideWaves = 4;
 constexpr int kWideTokens = 32;  // tokens per K/V tile
+constexpr int kWideBuffers = 4;  // ring depth
 
 template <int kD>
-constexpr int wide_lds_bytes() {
-  // two buffers x (K tile + V tile) x 32 tokens x padded row; the same bytes hold the rotated
-  // query tile (128 rows) before streaming starts
-  return 2 * 2 * kWideTokens * (kD / 8 + 1) * 16;
+struct WideShape {
+  static constexpr int kChunks = kD / 8;     // 16-byte pieces of a head row
+  static constexpr int kSteps = kD / 16;     // contraction steps of K.Q^T (32x32x16)
+  static constexpr int kDimTiles = kD / 32;  // 32-dim tiles of the output = dims a lane owns per V token
+  static constexpr int kVDw = kD / 64;       // dwords of a V token a lane reads
+  static constexpr int kRowBytes = kChunks * 16;
+  static constexpr int kRowsPerLoad = kWave / kChunks;              // tile rows one wave-level load covers
+  static constexpr int kLoadsPerKind = kWideTokens / kRowsPerLoad;  // loads per K (or V) tile
+  static constexpr int kLoadsPerWave = 2 * kLoadsPerKind / kWideWaves;
+  static constexpr int kTileBytes = kWideTokens * kRowBytes;  // a K (or V) tile
+  static constexpr int kBufferBytes = 2 * kTileBytes;
+  static constexpr int kLdsBytes = kWideBuffers * kBufferBytes;  // 128 KB at D = 256
+  // 32-row blocks per wave.  Two blocks halve the LDS bytes read per flop, but the state of a row
+  // (D fp32 accumulators + D 16-bit query elements) then fills the register file at D = 256:
+  // 64 rows need 256 + 128 of the 512 registers before any operand is staged, and the compiler
+  // spills.  D = 256 therefore runs one block per wave.
+  static constexpr int kBlocks = kD == 256 ? 1 : 2;
+  static constexpr int kWaveRows = 32 * kBlocks;
+  static constexpr int kTileRows = kWideWaves * kWaveRows;  // MFMA rows per workgroup
+  static_assert(128 * kRowBytes == 2 * kBufferBytes, "one row block of every wave fills two ring buffers");
+};
+
+template <int kD>
+__device__ __forceinline__ int wide_swz(int r) {
+  if constexpr (kD >= 128) return r & 15;
+  return (r >> 1) & 7;
+}
+
+// max over the two half-waves (lanes l and l ^ 32) without touching LDS
+__device__ __forceinline__ float half_wave_max(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
 template <typename E, int kD>
 __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArgs a) {
   using S = typename E::storage;
-  constexpr int kSteps = kD / 16;     // contraction steps of K.Q^T (32x32x16)
-  constexpr int kDimTiles = kD / 32;  // 32-dim tiles of the output = dims a lane owns per V token
-  constexpr int kChunks = kD / 8;     // 16-byte pieces of a head row
-  constexpr int kRow = kChunks + 1;   // padded LDS row, in 16-byte units
-  constexpr int kVDw = kD / 64;       // dwords of a V token a lane reads (D/32 dims)
+  using Sh = WideShape<kD>;
+  constexpr int kChunks = Sh::kChunks, kSteps = Sh::kSteps, kDimTiles = Sh::kDimTiles, kVDw = Sh::kVDw;
+  constexpr int kRowBytes = Sh::kRowBytes, kL = Sh::kLoadsPerWave, kB = Sh::kBlocks, kWaveRows = Sh::kWaveRows;
 
   extern __shared__ va_u32x4 smem[];
-  // buffer b: K tile at smem + b*2*32*kRow, V tile 32*kRow further
-  auto k_tile = [&](int b) __attribute__((always_inline)) { return smem + (b * 2) * kWideTokens * kRow; };
-  auto v_tile = [&](int b) __attribute__((always_inline)) { return smem + (b * 2 + 1) * kWideTokens * kRow; };
+  const char* lds = (const char*)smem;
 
   const ItemHead where = item_and_head(blockIdx.x, a.num_kv_heads);
   const int32_t* item = a.items + (long long)where.item * VA_ITEM_WORDS;
@@ -61,21 +90,46 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int lane = tid % kWave;
-  const int j = lane % 32;  // row within the wave's 32 rows / token within a tile / dim group
-  const int h = lane / 32;  // half-wave: contraction group
-  const int my_row = 32 * wave + j;
-  const int row_iq = my_row / G;
-  const int wave_iq_last = min(n_q - 1, (32 * wave + 31) / G);  // last tile row this wave serves
+  const int j = lane % 32;         // row within a 32-row block / token within a tile / dim group
+  const int h = lane / 32;         // half-wave: contraction group
+  const int row0 = kWaveRows * wave + j;  // this lane's row in block 0; block 1 is 32 further
+  int row_iq[kB];
+#pragma unroll
+  for (int b = 0; b < kB; ++b) row_iq[b] = (row0 + 32 * b) / G;
+  const bool wave_active = (kWaveRows * wave) / G < n_q;  // the wave owns real rows
   const S* kp = (const S*)a.k_pool + (long long)hk * kD;
   const S* vp = (const S*)a.v_pool + (long long)hk * kD;
   const int P = a.page_size;
+  const bool pow2_pages = (P & (P - 1)) == 0;
+  const int p_shift = __builtin_ctz(P);  // t / P and t % P as shift and mask (power-of-two pages)
+  const int row_bytes = (int)a.pool_row_stride * (int)sizeof(S);
 
-  float m_run = kNegBig, l_run = 0.f;
-  va_f32x16 o[kDimTiles];
+  // this lane's part of a wave-level load: row within the load and (swizzled) piece
+  const int ld_row0 = lane / kChunks;
+  const int ld_x0 = (lane % kChunks) ^ wide_swz<kD>(ld_row0);
+  // LDS offsets of what this lane reads from a tile
+  const int swz_j = wide_swz<kD>(j);
+  const int k_row_byte = j * kRowBytes;
+  int v_byte[8];  // token e of a 16-token step: (e / 4) * 8 + 4h + e % 4
 #pragma unroll
-  for (int t = 0; t < kDimTiles; ++t)
+  for (int e = 0; e < 8; ++e) {
+    const int tok = (e / 4) * 8 + 4 * h + (e % 4);
+    const int first_dim = j * (kD / 32);  // the lane's run of D/32 dims
+    v_byte[e] = tok * kRowBytes + 16 * ((first_dim / 8) ^ wide_swz<kD>(tok)) + 2 * (first_dim % 8);
+  }
+
+  float m_ref[kB], m_tile[kB], l_run[kB];  // reference maximum (log2 units), last tile maximum, row sum
+  va_f32x16 o[kB][kDimTiles];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
+  for (int b = 0; b < kB; ++b) {
+    m_ref[b] = kNegBig;
+    m_tile[b] = kNegBig;
+    l_run[b] = 0.f;
+#pragma unroll
+    for (int t = 0; t < kDimTiles; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[b][t][r] = 0.f;
+  }
 
   for (int li = 0; li < item[VA_I_N_LINKS]; ++li) {
     const int32_t* link = a.links + (long long)(item[VA_I_LINK_BEGIN] + li) * VA_LINK_WORDS;
@@ -86,211 +140,261 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     const int tok_end = link[VA_L_TOK_END];
     const int causal_base = link[VA_L_CAUSAL_BASE];
     const bool slots = lflags & VA_LINK_SLOTS;
-
-    // ---- rotate the whole query tile for this link into LDS (aliases the tile buffers) ----
-    __syncthreads();
-    for (int idx = tid; idx < kWideRows * kChunks; idx += kWideThreads) {
-      const int R = idx / kChunks, c = idx - R * kChunks;
-      const int iq = R / G, g = R - iq * G;
-      va_u32x4 packed = {0, 0, 0, 0};
-      if (iq < n_q) {
-        const int subrow = (lflags & VA_LINK_INDIRECT) ? a.qrefs[qref + iq] : qref + iq;
-        const long long src_row = a.sub_worker[subrow];
-        const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
-        const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
-        const uint4 piece = rotated_query_piece<E>(a.rope, qh, c * 8, p);
-        packed = va_u32x4{piece.x, piece.y, piece.z, piece.w};
-      }
-      smem[R * kRow + c] = packed;
-    }
-    __syncthreads();
-    va_u32x4 qf[kSteps];  // B operands: row my_row, dims [16s + 8h, +8)
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s) qf[s] = smem[my_row * kRow + 2 * s + h];
-    __syncthreads();
-
-    const int t_stop = min(tok_end, causal_base + n_q);             // tokens any row of the tile sees
-    const int t_row = min(tok_end, causal_base + row_iq + 1);       // tokens this lane's row sees
-    // tokens any row of this wave sees (none if the wave's rows lie beyond the tile)
-    const int t_wave = (32 * wave) / G < n_q ? min(tok_end, causal_base + wave_iq_last + 1) : -0x7fffffff;
-    const int t_last = t_stop - 1;
-    // tokens EVERY real row of this wave sees: tiles ending below it need no masking
-    const int t_wave_min = min(tok_end, causal_base + (32 * wave) / G + 1);
-
-    // global -> registers -> LDS.  Thread (ld_tok, ld_c) moves piece ld_c of tokens ld_tok + kTokStep*i of
-    // both the K and the V tile: rows are contiguous over threads, K and V share the row lookup.
-    constexpr int kTokStep = kWideThreads / kChunks;  // tokens per round of loads
-    constexpr int kRounds = kWideTokens / kTokStep;
-    const int ld_tok = tid / kChunks, ld_c = tid - ld_tok * kChunks;
     // a 16-token half tile lies inside one page only if the link starts on a 16-token boundary
-    const bool uniform_pages = !slots && (P % 16 == 0) && (tok_begin % 16 == 0);
-    va_u32x4 stage_k[kRounds], stage_v[kRounds];
-    auto fetch = [&](int t0) __attribute__((always_inline)) {
-      if (uniform_pages) {
-        // a 16-token half tile lies in one page: two wave-uniform page-table reads per tile
-        long long half_row[2];
+    const bool uniform_pages = !slots && pow2_pages && P >= 16 && (tok_begin % 16 == 0);
+
+    const int t_stop = min(tok_end, causal_base + n_q);  // tokens any row of the tile sees
+    const int t_last = t_stop - 1;
+    int t_row[kB];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const int t = min(t0 + 16 * u, t_last);
-          const int page = __builtin_amdgcn_readfirstlane(a.kv_indices[kv_begin + t / P]);
-          half_row[u] = (long long)page * P + ((t % P) & ~15);
-        }
-#pragma unroll
-        for (int i = 0; i < kRounds; ++i) {
-          const int tok = ld_tok + kTokStep * i;
-          const int t = min(t0 + tok, t_last);
-          const long long off = ((tok < 16 ? half_row[0] : half_row[1]) + (t & 15)) * a.pool_row_stride + 8 * ld_c;
-          stage_k[i] = *(const va_u32x4*)(kp + off);
-          stage_v[i] = *(const va_u32x4*)(vp + off);
-        }
-      } else {
-        long long off[kRounds];
-#pragma unroll
-        for (int i = 0; i < kRounds; ++i) {
-          const int t = min(t0 + ld_tok + kTokStep * i, t_last);
-          off[i] = kv_slot(a.kv_indices, kv_begin, t, P, slots) * a.pool_row_stride + 8 * ld_c;
-        }
-#pragma unroll
-        for (int i = 0; i < kRounds; ++i) {
-          stage_k[i] = *(const va_u32x4*)(kp + off[i]);
-          stage_v[i] = *(const va_u32x4*)(vp + off[i]);
-        }
-      }
+    for (int b = 0; b < kB; ++b) t_row[b] = min(tok_end, causal_base + row_iq[b] + 1);
+    // tokens any row of this wave sees, and tokens EVERY real row of it sees (no masking below that)
+    const int wave_iq_last = min(n_q - 1, (kWaveRows * wave + kWaveRows - 1) / G);
+    const int t_wave = wave_active ? min(tok_end, causal_base + wave_iq_last + 1) : -0x7fffffff;
+    const int t_wave_min = min(tok_end, causal_base + (kWaveRows * wave) / G + 1);
+    const int n_tiles = t_stop > tok_begin ? (t_stop - tok_begin + kWideTokens - 1) / kWideTokens : 0;
+
+    // Pool row of the 16-token group that holds token min(t0 + 16u, t_last) (uniform pages); read
+    // through the constant address space so that the lookup stays a scalar load.
+    auto group_row = [&](int t0, int u) __attribute__((always_inline)) {
+      const int t = min(t0 + 16 * u, t_last);
+      const int page = ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + (t >> p_shift)];
+      return ((long long)page << p_shift) + ((t & (P - 1)) & ~15);
     };
-    auto commit = [&](int b) __attribute__((always_inline)) {
-      va_u32x4* kt = k_tile(b);
-      va_u32x4* vt = v_tile(b);
+    // Request tile i into ring buffer i % kWideBuffers.  Rows past the visible range re-read the
+    // last visible token (their scores are masked).
+    auto issue_kind = [&](int i, auto uniform_tag, long long g0, long long g1) __attribute__((always_inline)) {
+      constexpr bool kUniform = decltype(uniform_tag)::value;
+      const int t0 = tok_begin + i * kWideTokens;
+      const char* buf = lds + (i % kWideBuffers) * Sh::kBufferBytes;
 #pragma unroll
-      for (int i = 0; i < kRounds; ++i) {
-        const int at = (ld_tok + kTokStep * i) * kRow + ld_c;
-        kt[at] = stage_k[i];
-        vt[at] = stage_v[i];
-      }
-    };
-
-    int t0 = tok_begin;
-    int buf = 0;
-    if (t0 < t_stop) {
-      fetch(t0);
-      commit(0);
-      __syncthreads();
-    }
-    for (; t0 < t_stop; t0 += kWideTokens) {
-      const bool more = t0 + kWideTokens < t_stop;
-#if VA_WIDE_EXPERIMENT != 1
-      if (more) fetch(t0 + kWideTokens);
-#endif
-
-#if VA_WIDE_EXPERIMENT == 2
-      if (false) {
-#else
-      if (t0 < t_wave) {
-#endif
-        const va_u32x4* kt = k_tile(buf);
-        const va_u32x4* vt = v_tile(buf);
-        // ---- scores.  K fragments are read from LDS in groups of four, two groups ahead of the
-        // MFMAs that consume them, so the matrix pipe never waits on an LDS round trip. ----
-        constexpr int kGroups = kSteps / 4;
-        va_u32x4 kfr[2][4];
-        auto read_group = [&](int g, va_u32x4 (&dst)[4]) __attribute__((always_inline)) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) dst[q] = kt[j * kRow + 2 * (4 * g + q) + h];
-        };
-        read_group(0, kfr[0]);
-        if constexpr (kGroups > 1) read_group(1, kfr[1]);
-        va_f32x16 sc;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sc[r] = 0.f;
-        __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs (the scheduler would sink them)
-#pragma unroll
-        for (int g = 0; g < kGroups; ++g) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) sc = Mma<E>::run32(kfr[g & 1][q], qf[4 * g + q], sc);
-          if (g + 2 < kGroups) read_group(g + 2, kfr[g & 1]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-
-        // ---- online softmax: reg r holds token t0 + (r/4)*8 + 4h + r%4 of row my_row.  Interior
-        // tiles (every row of the wave sees all 32 tokens) skip the masking; the scale is folded
-        // into the exponent: p = 2^(s*c - m). ----
-        float tile_max = -INFINITY;
-        if (t0 + kWideTokens <= t_wave_min) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) tile_max = fmaxf(tile_max, sc[r]);
+      for (int u = 0; u < kL; ++u) {
+        const int q = wave * kL + u;  // wave-uniform
+        const bool is_v = q >= Sh::kLoadsPerKind;
+        const int first_row = (is_v ? q - Sh::kLoadsPerKind : q) * Sh::kRowsPerLoad;
+        const int t = min(t0 + first_row + ld_row0, t_last);
+        const int piece = 16 * (ld_x0 ^ wide_swz<kD>(first_row));
+        const char* src;
+        if constexpr (kUniform) {
+          const long long group = first_row < 16 ? g0 : g1;  // wave-uniform
+          src = (const char*)(is_v ? vp : kp) + group * row_bytes + (uint32_t)((t & 15) * row_bytes + piece);
         } else {
+          src = (const char*)(is_v ? vp : kp) + kv_slot(a.kv_indices, kv_begin, t, P, slots) * row_bytes + piece;
+        }
+        const char* dst = buf + (is_v ? Sh::kTileBytes : 0) + first_row * kRowBytes;  // + 16 * lane, implied
+        load_to_lds(src, __builtin_amdgcn_readfirstlane(lds_address(dst)));
+      }
+    };
+    // one branch per tile on the kind of page table; the computation below exists once
+    auto issue = [&](int i, long long g0, long long g1) __attribute__((always_inline)) {
+      if (uniform_pages) {
+        issue_kind(i, std::true_type{}, g0, g1);
+      } else {
+        issue_kind(i, std::false_type{}, 0, 0);
+      }
+    };
+    auto issue_now = [&](int i) __attribute__((always_inline)) {
+      const int t0 = tok_begin + i * kWideTokens;
+      if (uniform_pages) {
+        issue(i, group_row(t0, 0), group_row(t0, 1));
+      } else {
+        issue(i, 0, 0);
+      }
+    };
+
+    // ---- set-up: first two tiles on their way, then the query tile (buffers 2 and 3) ----
+    __syncthreads();  // every wave is done with the previous link's buffers
+    if (0 < n_tiles) issue_now(0);
+    if (1 < n_tiles) issue_now(1);
+    va_u32x4* q_stage = (va_u32x4*)(lds + 2 * Sh::kBufferBytes);
+    va_u32x4 qf[kB][kSteps];  // B operands: row of block b, dims [16s + 8h, +8)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int t = t0 + (r / 4) * 8 + 4 * h + (r % 4);
-            sc[r] = t < t_row ? sc[r] : -INFINITY;
-            tile_max = fmaxf(tile_max, sc[r]);
+    for (int pass = 0; pass < kB; ++pass) {
+      for (int idx = tid; idx < 128 * kChunks; idx += kWideThreads) {
+        const int Rl = idx / kChunks, c = idx - Rl * kChunks;
+        const int R = kWaveRows * (Rl / 32) + 32 * pass + Rl % 32;  // block `pass` of every wave
+        const int iq = R / G, g = R - iq * G;
+        va_u32x4 packed = {0, 0, 0, 0};
+        if (iq < n_q) {
+          const int subrow = (lflags & VA_LINK_INDIRECT) ? a.qrefs[qref + iq] : qref + iq;
+          const long long src_row = a.sub_worker[subrow];
+          const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
+          const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
+          const uint4 piece = rotated_query_piece<E>(a.rope, qh, c * 8, p);
+          packed = va_u32x4{piece.x, piece.y, piece.z, piece.w};
+        }
+        q_stage[Rl * kChunks + (c ^ wide_swz<kD>(Rl))] = packed;
+      }
+      ring_barrier<kAnyInFlight>();
+      {
+        const int Rl = 32 * wave + j;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) qf[pass][s] = q_stage[Rl * kChunks + ((2 * s + h) ^ wide_swz<kD>(Rl))];
+      }
+      ring_barrier<kAnyInFlight>();  // staging rows may be overwritten now
+    }
+
+    // ---- the tile loop ----
+    // The softmax runs against a per-row REFERENCE maximum m_ref that is raised only when a
+    // tile's maximum exceeds it by more than kRaise (in log2 units): p = exp2(s - m_ref) then
+    // stays below 2^kRaise, harmless for the 16-bit P operand and the fp32 sums, and any
+    // consistent reference gives the same softmax.  Raising m_ref means rescaling the D fp32
+    // accumulators of every row, which is vector-ALU work on registers that otherwise only the
+    // matrix pipe touches; it happens on the first tile and then hardly ever, so it is kept out
+    // of the hot loop: the loop breaks, the accumulators are rescaled, and the loop resumes with
+    // the tile whose scores are already in registers.
+    constexpr float kRaise = 14.f;
+    if (2 < n_tiles) issue_now(2);
+    va_f32x16 sc[kB];
+    bool resume = false;  // sc holds the scores of tile i; its barrier and refill are done
+    int i = 0;
+    while (i < n_tiles) {
+      for (; i < n_tiles; ++i) {
+        const int t0 = tok_begin + i * kWideTokens;
+        const char* kt = lds + (i % kWideBuffers) * Sh::kBufferBytes;
+        const char* vt = kt + Sh::kTileBytes;
+        if (!resume) {
+          const bool refill = i + 3 < n_tiles;
+          long long g0 = 0, g1 = 0;  // looked up before the barrier: the latency hides behind the wait
+          if (uniform_pages && refill) {
+            g0 = group_row(t0 + 3 * kWideTokens, 0);
+            g1 = group_row(t0 + 3 * kWideTokens, 1);
+          }
+          // This wave's loads of tile i have landed once only those of the (up to two) tiles
+          // requested after it are outstanding; the barrier then covers the other waves' loads and
+          // tells that every wave is done with tile i - 1, whose buffer tile i + 3 may now take.
+          if (i + 2 < n_tiles) {
+            ring_barrier<2 * kL>();
+          } else if (i + 1 < n_tiles) {
+            ring_barrier<kL>();
+          } else {
+            ring_barrier<0>();
+          }
+          if (refill) issue(i + 3, g0, g1);
+          if (t0 >= t_wave) continue;  // no row of this wave sees the tile
+
+          // ---- scores of all row blocks; a K fragment is read once for all of them.  All K
+          // fragments of the tile are requested up front: the matrix pipe then never waits for an
+          // LDS round trip between two products. ----
+          va_u32x4 kf[kSteps];
+#pragma unroll
+          for (int s = 0; s < kSteps; ++s) kf[s] = *(const va_u32x4*)(kt + k_row_byte + 16 * ((2 * s + h) ^ swz_j));
+#pragma unroll
+          for (int b = 0; b < kB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sc[b][r] = 0.f;
+#pragma unroll
+          for (int s = 0; s < kSteps; ++s) {
+#pragma unroll
+            for (int b = 0; b < kB; ++b) sc[b] = Mma<E>::run32(kf[s], qf[b][s], sc[b]);
+          }
+          // mask and find the tile maxima; reg r of a block is token t0 + (r/4)*8 + 4h + r%4 of its row
+          const bool masked = t0 + kWideTokens > t_wave_min;
+          bool raise = false;
+#pragma unroll
+          for (int b = 0; b < kB; ++b) {
+            if (masked) {
+#pragma unroll
+              for (int r = 0; r < 16; ++r)
+                sc[b][r] = (t0 + (r / 4) * 8 + 4 * h + (r % 4)) < t_row[b] ? sc[b][r] : -INFINITY;
+            }
+            float tile_max = sc[b][0];
+#pragma unroll
+            for (int r = 1; r < 16; ++r) tile_max = fmaxf(tile_max, sc[b][r]);
+            tile_max = half_wave_max(tile_max);
+            m_tile[b] = tile_max * a.scale_log2;
+            raise = raise || m_tile[b] > m_ref[b] + kRaise;
+          }
+          if (__any(raise)) {
+            resume = true;
+            break;
           }
         }
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
-        const float m_new = fmaxf(m_run, tile_max * a.scale_log2);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        float psum = 0.f;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          sc[r] = __builtin_amdgcn_exp2f(fmaf(sc[r], a.scale_log2, -m_new));
-          psum += sc[r];
-        }
-        l_run = l_run * alpha + psum;
-        if (__any(alpha != 1.f)) {
-#pragma unroll
-          for (int t = 0; t < kDimTiles; ++t) o[t] *= alpha;
-        }
+        resume = false;
 
-        // ---- O^T += V^T . P^T over two 16-token steps ----
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-          const va_u32x4 pf = {Mma<E>::pack(sc[8 * kk + 0], sc[8 * kk + 1]), Mma<E>::pack(sc[8 * kk + 2], sc[8 * kk + 3]),
-                               Mma<E>::pack(sc[8 * kk + 4], sc[8 * kk + 5]), Mma<E>::pack(sc[8 * kk + 6], sc[8 * kk + 7])};
-          // the lane's 8 tokens of this step, D/32 dims each (dims j*D/32 ..)
-          uint32_t vraw[8][kVDw];
+        // ---- the V rows of the first token step are requested before the exponentials ----
+        uint32_t vraw[2][8][kVDw];
+        auto read_v = [&](int kk) __attribute__((always_inline)) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
-            const int tok = (2 * kk + e / 4) * 8 + 4 * h + (e % 4);
+            const char* at = vt + v_byte[e] + kk * 16 * kRowBytes;
             if constexpr (kVDw == 4) {
-              const va_u32x4 x = vt[tok * kRow + j];
-              vraw[e][0] = x[0]; vraw[e][1] = x[1]; vraw[e][2] = x[2]; vraw[e][3] = x[3];
+              const va_u32x4 x = *(const va_u32x4*)at;
+              vraw[kk][e][0] = x[0]; vraw[kk][e][1] = x[1]; vraw[kk][e][2] = x[2]; vraw[kk][e][3] = x[3];
             } else if constexpr (kVDw == 2) {
-              const uint2 x = ((const uint2*)(vt + tok * kRow))[j];
-              vraw[e][0] = x.x; vraw[e][1] = x.y;
+              const uint2 x = *(const uint2*)at;
+              vraw[kk][e][0] = x.x; vraw[kk][e][1] = x.y;
             } else {
-              vraw[e][0] = ((const uint32_t*)(vt + tok * kRow))[j];
+              vraw[kk][e][0] = *(const uint32_t*)at;
             }
           }
+        };
+        read_v(0);
+#pragma unroll
+        for (int b = 0; b < kB; ++b) {
+          float sum = 0.f;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            sc[b][r] = __builtin_amdgcn_exp2f(fmaf(sc[b][r], a.scale_log2, -m_ref[b]));
+            sum += sc[b][r];
+          }
+          l_run[b] += sum;
+        }
+
+        // ---- O^T += V^T . P^T over two 16-token steps; a transposed V fragment serves all blocks ----
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          va_u32x4 pf[kB];
+#pragma unroll
+          for (int b = 0; b < kB; ++b)
+            pf[b] = va_u32x4{Mma<E>::pack(sc[b][8 * kk + 0], sc[b][8 * kk + 1]), Mma<E>::pack(sc[b][8 * kk + 2], sc[b][8 * kk + 3]),
+                             Mma<E>::pack(sc[b][8 * kk + 4], sc[b][8 * kk + 5]), Mma<E>::pack(sc[b][8 * kk + 6], sc[b][8 * kk + 7])};
+          if (kk == 0) read_v(1);  // on its way while the first step's products run
 #pragma unroll
           for (int t = 0; t < kDimTiles; ++t) {
             const int w = t / 2;
             const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
-            const va_u32x4 vf = {__builtin_amdgcn_perm(vraw[1][w], vraw[0][w], sel), __builtin_amdgcn_perm(vraw[3][w], vraw[2][w], sel),
-                                 __builtin_amdgcn_perm(vraw[5][w], vraw[4][w], sel), __builtin_amdgcn_perm(vraw[7][w], vraw[6][w], sel)};
-            o[t] = Mma<E>::run32(vf, pf, o[t]);
+            const va_u32x4 vf = {__builtin_amdgcn_perm(vraw[kk][1][w], vraw[kk][0][w], sel), __builtin_amdgcn_perm(vraw[kk][3][w], vraw[kk][2][w], sel),
+                                 __builtin_amdgcn_perm(vraw[kk][5][w], vraw[kk][4][w], sel), __builtin_amdgcn_perm(vraw[kk][7][w], vraw[kk][6][w], sel)};
+#pragma unroll
+            for (int b = 0; b < kB; ++b) Mma<E>::run32_acc(vf, pf[b], o[b][t]);
           }
         }
       }
-
-#if VA_WIDE_EXPERIMENT != 1
-      if (more) commit(buf ^ 1);
-#endif
-      __syncthreads();
-      buf ^= 1;
+      if (resume) {
+        // raise the references to this tile's maxima and rescale what was accumulated against the old ones
+        accumulator_fence();
+#pragma unroll
+        for (int b = 0; b < kB; ++b) {
+          const float m_new = fmaxf(m_ref[b], m_tile[b]);
+          const float alpha = __builtin_amdgcn_exp2f(m_ref[b] - m_new);
+          m_ref[b] = m_new;
+          l_run[b] *= alpha;
+#pragma unroll
+          for (int t = 0; t < kDimTiles; ++t) o[b][t] *= alpha;
+        }
+      }
     }
   }
 
-  l_run += __shfl_xor(l_run, 32, kWave);
-
-  // ---- emit: accumulator reg r of dim tile T is dim ((r/4)*8 + 4h + r%4) * D/32 + T of row my_row ----
-  if (row_iq < n_q) {
-    const int g = my_row - row_iq * G;
+  accumulator_fence();
+  // ---- emit: accumulator reg r of dim tile T is dim ((r/4)*8 + 4h + r%4) * D/32 + T of the lane's row ----
+#pragma unroll
+  for (int b = 0; b < kB; ++b) {
+    float l = l_run[b];
+    {
+      const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(l), __float_as_uint(l), false, false);
+      l = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
+    const int my_row = row0 + 32 * b;
+    const int iq = row_iq[b];
+    if (iq >= n_q) continue;
+    const int g = my_row - iq * G;
     const int hq = hk * G + g;
-    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    const float inv = l > 0.f ? 1.f / l : 0.f;
     if (part_base < 0) {
       const int32_t* link0 = a.links + (long long)item[VA_I_LINK_BEGIN] * VA_LINK_WORDS;
-      const int subrow =
-          (link0[VA_L_FLAGS] & VA_LINK_INDIRECT) ? a.qrefs[link0[VA_L_QREF] + row_iq] : link0[VA_L_QREF] + row_iq;
+      const int subrow = (link0[VA_L_FLAGS] & VA_LINK_INDIRECT) ? a.qrefs[link0[VA_L_QREF] + iq] : link0[VA_L_QREF] + iq;
       const long long out_row = a.sub_worker[subrow];
       S* orow = (S*)a.out + (out_row * a.num_q_heads + hq) * (long long)kD;
 #pragma unroll
@@ -298,7 +402,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         const int d0 = ((r / 4) * 8 + 4 * h + (r % 4)) * kDimTiles;
         uint32_t w[kDimTiles / 2];
 #pragma unroll
-        for (int t = 0; t < kDimTiles / 2; ++t) w[t] = Mma<E>::pack(o[2 * t][r] * inv, o[2 * t + 1][r] * inv);
+        for (int t = 0; t < kDimTiles / 2; ++t) w[t] = Mma<E>::pack(o[b][2 * t][r] * inv, o[b][2 * t + 1][r] * inv);
         if constexpr (kDimTiles == 8) {
           *(uint4*)(orow + d0) = make_uint4(w[0], w[1], w[2], w[3]);
         } else if constexpr (kDimTiles == 4) {
@@ -308,21 +412,21 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         }
       }
       if (h == 0 && a.lse) {
-        const float lse2 = l_run > 0.f ? m_run + log2f(l_run) : -INFINITY;
+        const float lse2 = l > 0.f ? m_ref[b] + log2f(l) : -INFINITY;
         a.lse[out_row * a.num_q_heads + hq] = a.lse_base2 ? lse2 : lse2 * kLn2;
       }
     } else {
-      const long long slot = (long long)(part_base + row_iq) * a.num_q_heads + hq;
+      const long long slot = (long long)(part_base + iq) * a.num_q_heads + hq;
       float* prow = a.part_acc + slot * kD;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int d0 = ((r / 4) * 8 + 4 * h + (r % 4)) * kDimTiles;
 #pragma unroll
-        for (int t = 0; t < kDimTiles; ++t) prow[d0 + t] = o[t][r];
+        for (int t = 0; t < kDimTiles; ++t) prow[d0 + t] = o[b][t][r];
       }
       if (h == 0) {
-        a.part_ml[slot * 2 + 0] = m_run;
-        a.part_ml[slot * 2 + 1] = l_run;
+        a.part_ml[slot * 2 + 0] = m_ref[b];
+        a.part_ml[slot * 2 + 1] = l;
       }
     }
   }
@@ -330,7 +434,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
 
 template <typename E, int kD>
 static int launch_wide_one(const AttnArgs& a, int n_items, hipStream_t stream) {
-  constexpr int bytes = wide_lds_bytes<kD>();
+  constexpr int bytes = WideShape<kD>::kLdsBytes;
   static bool configured = false;  // raising the limit is idempotent; a race only repeats the call
   if (!configured) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mfma_wide_kernel<E, kD>),

@@ -112,9 +112,9 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   // wide kernel, whose four waves share every K/V tile through LDS.
   int wide_tile = 0;
   if (kernel == VA_KERNEL_MFMA && !(params && params->wide_tile < 0)) {
-    wide_tile = params && params->wide_tile > 0 ? params->wide_tile : va_mfma_wide_q_tile(g);
-    if (wide_tile > va_mfma_wide_q_tile(g))
-      return va_fail(VA_ERR_ARG, "wide_tile %d exceeds the kernel's maximum %d", wide_tile, va_mfma_wide_q_tile(g));
+    wide_tile = params && params->wide_tile > 0 ? params->wide_tile : va_mfma_wide_q_tile(g, shape->head_dim);
+    if (wide_tile > va_mfma_wide_q_tile(g, shape->head_dim))
+      return va_fail(VA_ERR_ARG, "wide_tile %d exceeds the kernel's maximum %d", wide_tile, va_mfma_wide_q_tile(g, shape->head_dim));
     if (wide_tile <= q_tile) wide_tile = 0;
   }
   // Cut n query rows into tiles: wide ones while more than q_tile rows remain, then narrow ones.

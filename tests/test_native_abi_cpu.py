@@ -203,7 +203,7 @@ def test_matrix_core_plans_with_wide_tiles_cover_every_pair_once(seed, prefill, 
                                   kernel=native.VA_KERNEL_MFMA, wide_tile=wide_tile, kv_chunk=rng.choice([0, 64]))
     assert rc == 0, native.lib.va_last_error()
     assert counts.kernel == native.VA_KERNEL_MFMA and counts.q_tile == 4
-    assert counts.wide_tile == {0: 32, 8: 8, -1: 0}[wide_tile]
+    assert counts.wide_tile == {0: 64, 8: 8, -1: 0}[wide_tile]
     h, items, *_ = decode_plan(blob)
     kinds = [int(i[5]) for i in items]
     assert kinds == sorted(kinds, reverse=True) and sum(kinds) == counts.n_wide_items == h[H["N_WIDE"]]
