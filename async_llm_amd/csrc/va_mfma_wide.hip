@@ -165,7 +165,11 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     // last visible token (their scores are masked).
     auto issue_kind = [&](int i, auto uniform_tag, long long g0, long long g1) __attribute__((always_inline)) {
       constexpr bool kUniform = decltype(uniform_tag)::value;
+#if VA_WIDE_EXPERIMENT == 7
+      const int t0 = tok_begin;  // every tile re-reads the first one: cache hits only
+#else
       const int t0 = tok_begin + i * kWideTokens;
+#endif
       const char* buf = lds + (i % kWideBuffers) * Sh::kBufferBytes;
 #pragma unroll
       for (int u = 0; u < kL; ++u) {
@@ -257,8 +261,13 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
           const bool refill = i + 3 < n_tiles;
           long long g0 = 0, g1 = 0;  // looked up before the barrier: the latency hides behind the wait
           if (uniform_pages && refill) {
+#if VA_WIDE_EXPERIMENT == 7
+            g0 = group_row(tok_begin, 0);
+            g1 = group_row(tok_begin, 1);
+#else
             g0 = group_row(t0 + 3 * kWideTokens, 0);
             g1 = group_row(t0 + 3 * kWideTokens, 1);
+#endif
           }
           // This wave's loads of tile i have landed once only those of the (up to two) tiles
           // requested after it are outstanding; the barrier then covers the other waves' loads and
@@ -270,8 +279,13 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
           } else {
             ring_barrier<0>();
           }
+#if VA_WIDE_EXPERIMENT != 5 && VA_WIDE_EXPERIMENT != 6
           if (refill) issue(i + 3, g0, g1);
+#endif
           if (t0 >= t_wave) continue;  // no row of this wave sees the tile
+#if VA_WIDE_EXPERIMENT == 1 || VA_WIDE_EXPERIMENT == 6 || VA_WIDE_EXPERIMENT == 7
+          continue;
+#endif
 
           // ---- scores of all row blocks; a K fragment is read once for all of them.  All K
           // fragments of the tile are requested up front: the matrix pipe then never waits for an
@@ -288,6 +302,10 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
 #pragma unroll
             for (int b = 0; b < kB; ++b) sc[b] = Mma<E>::run32(kf[s], qf[b][s], sc[b]);
           }
+#if VA_WIDE_EXPERIMENT == 2
+          l_run[0] += sc[0][0] + sc[kB - 1][5];
+          continue;
+#endif
           // mask and find the tile maxima; reg r of a block is token t0 + (r/4)*8 + 4h + r%4 of its row
           const bool masked = t0 + kWideTokens > t_wave_min;
           bool raise = false;
@@ -341,6 +359,9 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
           l_run[b] += sum;
         }
 
+#if VA_WIDE_EXPERIMENT == 3
+        continue;
+#endif
         // ---- O^T += V^T . P^T over two 16-token steps; a transposed V fragment serves all blocks ----
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
