@@ -27,12 +27,22 @@ struct Mma<BF16> {
   }
   // Same product with the accumulator pinned in the accumulation registers (AGPRs).  Written as
   // assembly because the register allocator otherwise treats AGPRs as spill space for a long-lived
-  // accumulator and copies all of it to VGPRs and back around every tile.  The leading s_nop covers
-  // the wait states between the vector ALU writing an operand and the matrix pipe reading it, which
-  // the compiler cannot insert for code it does not see; callers wait (accumulator_fence) before
-  // reading the accumulator with anything but another product.
+  // accumulator and copies all of it to VGPRs and back around every tile.  The compiler cannot
+  // insert wait states for code it does not see: the leading s_nop covers the two wait states
+  // between a vector-ALU write of an operand (the transposed V fragment, the packed P) and the
+  // matrix pipe reading it, and callers wait (accumulator_fence) before reading the accumulator
+  // with anything but another product.
   static __device__ __forceinline__ void run32_acc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  // The same with the accumulator in ordinary vector registers (for results the vector ALU reads
+  // next, the scores); `first`: the sum starts from zero.  No leading s_nop: the operands of these
+  // products come from LDS reads and from registers written long before.
+  static __device__ __forceinline__ void run32_vacc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void run32_vacc_first(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
   }
   template <typename A, typename B>
   static __device__ __forceinline__ va_f32x4 run(const A& a, const B& b, va_f32x4 c) {
@@ -58,6 +68,12 @@ struct Mma<F16> {
   }
   static __device__ __forceinline__ void run32_acc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void run32_vacc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void run32_vacc_first(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
   }
   template <typename A, typename B>
   static __device__ __forceinline__ va_f32x4 run(const A& a, const B& b, va_f32x4 c) {
@@ -128,6 +144,13 @@ constexpr int kAnyInFlight = 63;  // vmcnt(63): no wait on vector memory at all
 __device__ __forceinline__ void load_to_lds(const void* src, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base)
                : "memory");  // M0 is scratch for the compiler too: it sets it right before each use of its own
+}
+// The same with a wave-uniform base address and a 32-bit per-lane byte offset (no vector ALU work
+// to form 64-bit addresses).
+__device__ __forceinline__ void load_to_lds(const void* base, uint32_t lane_offset, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base),
+               "s"(lds_base)
+               : "memory");
 }
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;

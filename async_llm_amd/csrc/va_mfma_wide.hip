@@ -107,6 +107,12 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   // this lane's part of a wave-level load: row within the load and (swizzled) piece
   const int ld_row0 = lane / kChunks;
   const int ld_x0 = (lane % kChunks) ^ wide_swz<kD>(ld_row0);
+  // byte offset, from the first row of its 16-token group, of what this lane fetches in load u of a
+  // tile that lies entirely inside the visible range (uniform pages)
+  uint32_t ld_off[kL];
+#pragma unroll
+  for (int u = 0; u < kL; ++u)
+    ld_off[u] = (uint32_t)((u * Sh::kRowsPerLoad + ld_row0) * row_bytes + 16 * (ld_x0 ^ wide_swz<kD>(u * Sh::kRowsPerLoad)));
   // LDS offsets of what this lane reads from a tile
   const int swz_j = wide_swz<kD>(j);
   const int k_row_byte = j * kRowBytes;
@@ -154,59 +160,48 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     const int t_wave_min = min(tok_end, causal_base + (kWaveRows * wave) / G + 1);
     const int n_tiles = t_stop > tok_begin ? (t_stop - tok_begin + kWideTokens - 1) / kWideTokens : 0;
 
-    // Pool row of the 16-token group that holds token min(t0 + 16u, t_last) (uniform pages); read
-    // through the constant address space so that the lookup stays a scalar load.
-    auto group_row = [&](int t0, int u) __attribute__((always_inline)) {
-      const int t = min(t0 + 16 * u, t_last);
+    // Loads of a tile.  Wave w fetches one 16-token half of the K tile (w = 0, 1) or of the V tile
+    // (w = 2, 3): kL wave-level loads of kRowsPerLoad rows each.  With uniform pages the half lies
+    // in one page, so the wave needs ONE scalar page lookup per tile and every load is a
+    // wave-uniform base plus a per-lane offset that never changes (ld_off); tiles that reach past
+    // the visible range, and page tables with pages under 16 tokens or slot lists, look every
+    // row up per lane instead (rows past the range re-read the last visible token; their scores
+    // are masked).
+    const bool wave_is_v = wave >= 2;
+    const int wave_half = wave & 1;
+    const char* wave_pool = (const char*)(wave_is_v ? vp : kp);
+    const uint32_t wave_lds = __builtin_amdgcn_readfirstlane(lds_address(lds)) + (wave_is_v ? Sh::kTileBytes : 0) +
+                              wave_half * 16 * kRowBytes;
+    // pool row of this wave's half of tile i (uniform pages, tile inside the visible range); read
+    // through the constant address space so that the lookup stays a scalar load
+    auto half_row = [&](int i) __attribute__((always_inline)) {
+      const int t = tok_begin + i * kWideTokens + 16 * wave_half;
       const int page = ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + (t >> p_shift)];
-      return ((long long)page << p_shift) + ((t & (P - 1)) & ~15);
+      return ((long long)page << p_shift) + (t & (P - 1));
     };
-    // Request tile i into ring buffer i % kWideBuffers.  Rows past the visible range re-read the
-    // last visible token (their scores are masked).
-    auto issue_kind = [&](int i, auto uniform_tag, long long g0, long long g1) __attribute__((always_inline)) {
-      constexpr bool kUniform = decltype(uniform_tag)::value;
-#if VA_WIDE_EXPERIMENT == 7
-      const int t0 = tok_begin;  // every tile re-reads the first one: cache hits only
-#else
-      const int t0 = tok_begin + i * kWideTokens;
-#endif
-      const char* buf = lds + (i % kWideBuffers) * Sh::kBufferBytes;
+    auto tile_is_plain = [&](int i) __attribute__((always_inline)) {
+      return uniform_pages && tok_begin + (i + 1) * kWideTokens - 1 <= t_last;
+    };
+    auto issue = [&](int i, long long row) __attribute__((always_inline)) {
+      const uint32_t dst = wave_lds + (i % kWideBuffers) * Sh::kBufferBytes;
+      if (tile_is_plain(i)) {
+        const char* base = wave_pool + row * row_bytes;
 #pragma unroll
-      for (int u = 0; u < kL; ++u) {
-        const int q = wave * kL + u;  // wave-uniform
-        const bool is_v = q >= Sh::kLoadsPerKind;
-        const int first_row = (is_v ? q - Sh::kLoadsPerKind : q) * Sh::kRowsPerLoad;
-        const int t = min(t0 + first_row + ld_row0, t_last);
-        const int piece = 16 * (ld_x0 ^ wide_swz<kD>(first_row));
-        const char* src;
-        if constexpr (kUniform) {
-          const long long group = first_row < 16 ? g0 : g1;  // wave-uniform
-          src = (const char*)(is_v ? vp : kp) + group * row_bytes + (uint32_t)((t & 15) * row_bytes + piece);
-        } else {
-          src = (const char*)(is_v ? vp : kp) + kv_slot(a.kv_indices, kv_begin, t, P, slots) * row_bytes + piece;
+        for (int u = 0; u < kL; ++u) load_to_lds(base, ld_off[u], dst + u * 1024);
+      } else {
+        const int t0 = tok_begin + i * kWideTokens + 16 * wave_half;
+#pragma unroll
+        for (int u = 0; u < kL; ++u) {
+          const int r = u * Sh::kRowsPerLoad + ld_row0;
+          const int t = min(t0 + r, t_last);
+          const int piece = 16 * (ld_x0 ^ wide_swz<kD>(u * Sh::kRowsPerLoad));
+          load_to_lds(wave_pool + kv_slot(a.kv_indices, kv_begin, t, P, slots) * row_bytes + piece, dst + u * 1024);
         }
-        const char* dst = buf + (is_v ? Sh::kTileBytes : 0) + first_row * kRowBytes;  // + 16 * lane, implied
-        load_to_lds(src, __builtin_amdgcn_readfirstlane(lds_address(dst)));
       }
     };
-    // one branch per tile on the kind of page table; the computation below exists once
-    auto issue = [&](int i, long long g0, long long g1) __attribute__((always_inline)) {
-      if (uniform_pages) {
-        issue_kind(i, std::true_type{}, g0, g1);
-      } else {
-        issue_kind(i, std::false_type{}, 0, 0);
-      }
-    };
-    auto issue_now = [&](int i) __attribute__((always_inline)) {
-      const int t0 = tok_begin + i * kWideTokens;
-      if (uniform_pages) {
-        issue(i, group_row(t0, 0), group_row(t0, 1));
-      } else {
-        issue(i, 0, 0);
-      }
-    };
+    auto issue_now = [&](int i) __attribute__((always_inline)) { issue(i, tile_is_plain(i) ? half_row(i) : 0); };
 
-    // ---- set-up: first two tiles on their way, then the query tile (buffers 2 and 3) ----
+    // ---- set-up: first two tiles on their way, then the query tile (staged in buffers 2 and 3) ----
     __syncthreads();  // every wave is done with the previous link's buffers
     if (0 < n_tiles) issue_now(0);
     if (1 < n_tiles) issue_now(1);
@@ -239,73 +234,88 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     }
 
     // ---- the tile loop ----
-    // The softmax runs against a per-row REFERENCE maximum m_ref that is raised only when a
-    // tile's maximum exceeds it by more than kRaise (in log2 units): p = exp2(s - m_ref) then
-    // stays below 2^kRaise, harmless for the 16-bit P operand and the fp32 sums, and any
-    // consistent reference gives the same softmax.  Raising m_ref means rescaling the D fp32
-    // accumulators of every row, which is vector-ALU work on registers that otherwise only the
-    // matrix pipe touches; it happens on the first tile and then hardly ever, so it is kept out
-    // of the hot loop: the loop breaks, the accumulators are rescaled, and the loop resumes with
-    // the tile whose scores are already in registers.
+    // Reference maximum.  The softmax runs against a per-row REFERENCE maximum m_ref that is
+    // raised only when a tile's maximum exceeds it by more than kRaise (in log2 units):
+    // p = exp2(s - m_ref) then stays below 2^kRaise, harmless for the 16-bit P operand and the
+    // fp32 sums, and any consistent reference gives the same softmax.  Raising m_ref means
+    // rescaling the D fp32 accumulators of every row, vector-ALU work on registers that otherwise
+    // only the matrix pipe touches; it happens on the first tile and then hardly ever, so it is
+    // kept out of the hot loop: the loop breaks, the accumulators are rescaled, the loop resumes.
+    //
+    // Software pipeline.  One wave per SIMD means nothing but this wave's own instruction order
+    // can keep the matrix pipe busy, so the loop body is written as pieces pinned in order with
+    // scheduling barriers: while the scores of tile i+1 are computed (matrix pipe), the
+    // exponentials of tile i run on the vector ALU; while the products P.V of tile i run, the V
+    // fragments of the next product are transposed.
+    //
+    // Ring.  ring_step(k): wait until tile k has landed for the whole workgroup (one barrier) and
+    // request tile k + 2 into the buffer of tile k - 2, which every wave has left by then.  Every
+    // wave makes every step exactly once, in order; a step is made just before tile k is first
+    // needed (its K, for the scores computed one iteration ahead).
     constexpr float kRaise = 14.f;
-    if (2 < n_tiles) issue_now(2);
-    va_f32x16 sc[kB];
-    bool resume = false;  // sc holds the scores of tile i; its barrier and refill are done
-    int i = 0;
-    while (i < n_tiles) {
-      for (; i < n_tiles; ++i) {
-        const int t0 = tok_begin + i * kWideTokens;
-        const char* kt = lds + (i % kWideBuffers) * Sh::kBufferBytes;
-        const char* vt = kt + Sh::kTileBytes;
-        if (!resume) {
-          const bool refill = i + 3 < n_tiles;
-          long long g0 = 0, g1 = 0;  // looked up before the barrier: the latency hides behind the wait
-          if (uniform_pages && refill) {
-#if VA_WIDE_EXPERIMENT == 7
-            g0 = group_row(tok_begin, 0);
-            g1 = group_row(tok_begin, 1);
+#if VA_WIDE_EXPERIMENT == 1  // ring only
+    const int n_vis = 0;
 #else
-            g0 = group_row(t0 + 3 * kWideTokens, 0);
-            g1 = group_row(t0 + 3 * kWideTokens, 1);
+    const int n_vis = t_wave > tok_begin ? min(n_tiles, (t_wave - tok_begin + kWideTokens - 1) / kWideTokens) : 0;
 #endif
-          }
-          // This wave's loads of tile i have landed once only those of the (up to two) tiles
-          // requested after it are outstanding; the barrier then covers the other waves' loads and
-          // tells that every wave is done with tile i - 1, whose buffer tile i + 3 may now take.
-          if (i + 2 < n_tiles) {
-            ring_barrier<2 * kL>();
-          } else if (i + 1 < n_tiles) {
-            ring_barrier<kL>();
-          } else {
-            ring_barrier<0>();
-          }
-#if VA_WIDE_EXPERIMENT != 5 && VA_WIDE_EXPERIMENT != 6
-          if (refill) issue(i + 3, g0, g1);
+    int next_step = 0;
+    auto ring_step = [&]() __attribute__((always_inline)) {
+      const int k = next_step++;
+      const bool refill = k + 2 < n_tiles;
+      long long row = 0;  // looked up before the barrier: the latency hides behind the wait
+      if (refill && tile_is_plain(k + 2)) row = half_row(k + 2);
+      if (k + 1 < n_tiles) {
+        ring_barrier<kL>();  // only the loads of tile k + 1 may still be outstanding
+      } else {
+        ring_barrier<0>();
+      }
+#if VA_WIDE_EXPERIMENT != 5 && VA_WIDE_EXPERIMENT != 8  // 5, 8: computation only
+      if (refill) issue(k + 2, row);
 #endif
-          if (t0 >= t_wave) continue;  // no row of this wave sees the tile
-#if VA_WIDE_EXPERIMENT == 1 || VA_WIDE_EXPERIMENT == 6 || VA_WIDE_EXPERIMENT == 7
-          continue;
-#endif
+    };
 
-          // ---- scores of all row blocks; a K fragment is read once for all of them.  All K
-          // fragments of the tile are requested up front: the matrix pipe then never waits for an
-          // LDS round trip between two products. ----
-          va_u32x4 kf[kSteps];
+    va_f32x16 sc[kB];       // scores, then probabilities, of the current tile
+    va_f32x16 sc_next[kB];  // scores of the next tile, accumulating
+    va_u32x4 kf[kSteps];
+    auto read_k = [&](int tile) __attribute__((always_inline)) {
+      const char* kt = lds + (tile % kWideBuffers) * Sh::kBufferBytes;
+#if VA_WIDE_EXPERIMENT == 8  // no LDS reads: one fragment stands in for all
+      kf[0] = *(const va_u32x4*)(kt + k_row_byte);
 #pragma unroll
-          for (int s = 0; s < kSteps; ++s) kf[s] = *(const va_u32x4*)(kt + k_row_byte + 16 * ((2 * s + h) ^ swz_j));
-#pragma unroll
-          for (int b = 0; b < kB; ++b)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) sc[b][r] = 0.f;
-#pragma unroll
-          for (int s = 0; s < kSteps; ++s) {
-#pragma unroll
-            for (int b = 0; b < kB; ++b) sc[b] = Mma<E>::run32(kf[s], qf[b][s], sc[b]);
-          }
-#if VA_WIDE_EXPERIMENT == 2
-          l_run[0] += sc[0][0] + sc[kB - 1][5];
-          continue;
+      for (int s = 1; s < kSteps; ++s) kf[s] = kf[0] + (uint32_t)s;
+      return;
 #endif
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) kf[s] = *(const va_u32x4*)(kt + k_row_byte + 16 * ((2 * s + h) ^ swz_j));
+    };
+    auto score_step = [&](int s) __attribute__((always_inline)) {
+#pragma unroll
+      for (int b = 0; b < kB; ++b) {
+        if (s == 0) {
+          Mma<E>::run32_vacc_first(kf[s], qf[b][s], sc_next[b]);
+        } else {
+          Mma<E>::run32_vacc(kf[s], qf[b][s], sc_next[b]);
+        }
+      }
+    };
+
+    if (n_vis > 0) {  // scores of tile 0
+      ring_step();
+      read_k(0);
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) score_step(s);
+      accumulator_fence();
+#pragma unroll
+      for (int b = 0; b < kB; ++b) sc[b] = sc_next[b];
+    }
+    bool resume = false;  // the step for tile i + 1 is made and sc holds the (masked) scores of tile i
+    int i = 0;
+    while (i < n_vis) {
+      for (; i < n_vis; ++i) {
+        const int t0 = tok_begin + i * kWideTokens;
+        const bool has_next = i + 1 < n_vis;
+        if (!resume) {
+          if (i + 1 < n_tiles) ring_step();  // tile i + 1 has landed
           // mask and find the tile maxima; reg r of a block is token t0 + (r/4)*8 + 4h + r%4 of its row
           const bool masked = t0 + kWideTokens > t_wave_min;
           bool raise = false;
@@ -330,12 +340,16 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         }
         resume = false;
 
-        // ---- the V rows of the first token step are requested before the exponentials ----
+        const char* vt = lds + (i % kWideBuffers) * Sh::kBufferBytes + Sh::kTileBytes;
         uint32_t vraw[2][8][kVDw];
         auto read_v = [&](int kk) __attribute__((always_inline)) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
+#if VA_WIDE_EXPERIMENT == 8
+            const char* at = vt + v_byte[0];
+#else
             const char* at = vt + v_byte[e] + kk * 16 * kRowBytes;
+#endif
             if constexpr (kVDw == 4) {
               const va_u32x4 x = *(const va_u32x4*)at;
               vraw[kk][e][0] = x[0]; vraw[kk][e][1] = x[1]; vraw[kk][e][2] = x[2]; vraw[kk][e][3] = x[3];
@@ -347,39 +361,68 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
             }
           }
         };
-        read_v(0);
+        // ---- phase A: scores of tile i + 1 (matrix pipe) under the exponentials of tile i ----
+        float sum[kB];
 #pragma unroll
-        for (int b = 0; b < kB; ++b) {
-          float sum = 0.f;
+        for (int b = 0; b < kB; ++b) sum[b] = 0.f;
+        auto exp_piece = [&](int r) __attribute__((always_inline)) {
+#pragma unroll
+          for (int b = 0; b < kB; ++b) {
+            sc[b][r] = __builtin_amdgcn_exp2f(fmaf(sc[b][r], a.scale_log2, -m_ref[b]));
+            sum[b] += sc[b][r];
+          }
+        };
+        constexpr int kPiecesPerStep = 16 / kSteps > 0 ? 16 / kSteps : 1;  // exponentials between two score steps
+        if (has_next) {
+          read_k(i + 1);
+          read_v(0);
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            sc[b][r] = __builtin_amdgcn_exp2f(fmaf(sc[b][r], a.scale_log2, -m_ref[b]));
-            sum += sc[b][r];
+            if (r % kPiecesPerStep == 0) score_step(r / kPiecesPerStep);
+            __builtin_amdgcn_sched_barrier(0);
+            exp_piece(r);
+            __builtin_amdgcn_sched_barrier(0);
           }
-          l_run[b] += sum;
-        }
-
-#if VA_WIDE_EXPERIMENT == 3
-        continue;
-#endif
-        // ---- O^T += V^T . P^T over two 16-token steps; a transposed V fragment serves all blocks ----
+        } else {
+          read_v(0);
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-          va_u32x4 pf[kB];
+          for (int r = 0; r < 16; ++r) exp_piece(r);
+        }
+#pragma unroll
+        for (int b = 0; b < kB; ++b) l_run[b] += sum[b];
+
+        // ---- phase B: O^T += V^T . P^T over two 16-token steps; while a product runs, the V
+        // fragment of the next one is transposed; a transposed fragment serves all row blocks ----
+        read_v(1);
+        va_u32x4 pf[2][kB];
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
           for (int b = 0; b < kB; ++b)
-            pf[b] = va_u32x4{Mma<E>::pack(sc[b][8 * kk + 0], sc[b][8 * kk + 1]), Mma<E>::pack(sc[b][8 * kk + 2], sc[b][8 * kk + 3]),
-                             Mma<E>::pack(sc[b][8 * kk + 4], sc[b][8 * kk + 5]), Mma<E>::pack(sc[b][8 * kk + 6], sc[b][8 * kk + 7])};
-          if (kk == 0) read_v(1);  // on its way while the first step's products run
+            pf[kk][b] = va_u32x4{Mma<E>::pack(sc[b][8 * kk + 0], sc[b][8 * kk + 1]), Mma<E>::pack(sc[b][8 * kk + 2], sc[b][8 * kk + 3]),
+                                 Mma<E>::pack(sc[b][8 * kk + 4], sc[b][8 * kk + 5]), Mma<E>::pack(sc[b][8 * kk + 6], sc[b][8 * kk + 7])};
+        auto transposed = [&](int idx) __attribute__((always_inline)) {
+          const int kk = idx / kDimTiles, t = idx % kDimTiles;
+          const int w = t / 2;
+          const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
+          return va_u32x4{__builtin_amdgcn_perm(vraw[kk][1][w], vraw[kk][0][w], sel), __builtin_amdgcn_perm(vraw[kk][3][w], vraw[kk][2][w], sel),
+                          __builtin_amdgcn_perm(vraw[kk][5][w], vraw[kk][4][w], sel), __builtin_amdgcn_perm(vraw[kk][7][w], vraw[kk][6][w], sel)};
+        };
+        va_u32x4 vf = transposed(0);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int t = 0; t < kDimTiles; ++t) {
-            const int w = t / 2;
-            const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
-            const va_u32x4 vf = {__builtin_amdgcn_perm(vraw[kk][1][w], vraw[kk][0][w], sel), __builtin_amdgcn_perm(vraw[kk][3][w], vraw[kk][2][w], sel),
-                                 __builtin_amdgcn_perm(vraw[kk][5][w], vraw[kk][4][w], sel), __builtin_amdgcn_perm(vraw[kk][7][w], vraw[kk][6][w], sel)};
+        for (int idx = 0; idx < 2 * kDimTiles; ++idx) {
+          const int kk = idx / kDimTiles, t = idx % kDimTiles;
 #pragma unroll
-            for (int b = 0; b < kB; ++b) Mma<E>::run32_acc(vf, pf[b], o[b][t]);
-          }
+          for (int b = 0; b < kB; ++b) Mma<E>::run32_acc(vf, pf[kk][b], o[b][t]);
+          __builtin_amdgcn_sched_barrier(0);
+          if (idx + 1 < 2 * kDimTiles) vf = transposed(idx + 1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (has_next) {  // the scores of tile i + 1 were complete long before the last product
+#pragma unroll
+          for (int b = 0; b < kB; ++b) sc[b] = sc_next[b];
         }
       }
       if (resume) {
@@ -396,6 +439,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         }
       }
     }
+    while (next_step < n_tiles) ring_step();  // tiles this wave does not see: keep in step with the others
   }
 
   accumulator_fence();
