@@ -121,6 +121,47 @@ __device__ __forceinline__ uint4 rotated_query_piece(const RopeDev& rope, const 
   return make_uint4(out[0], out[1], out[2], out[3]);
 }
 
+// Two 16-byte pieces of a rotated query head row at once.  Unit x of a row (0 <= x < D/16) covers
+// the rotary pair of pieces (x, x + rotary_dim/16) -- both halves of the same eight rotations, so
+// the inputs, the cos/sin entries and the products are shared -- or, past the rotary part, two
+// adjacent pieces that pass through.  c0/c1 receive the piece indices.
+template <typename E>
+__device__ __forceinline__ void rotated_query_unit(const RopeDev& rope, const typename E::storage* qh, int x,
+                                                   const Pos3& p, int& c0, int& c1, uint4& o0, uint4& o1) {
+  using S = typename E::storage;
+  const int pair_units = rope.rotary_dim / 16;
+  if (x >= pair_units) {
+    c0 = rope.rotary_dim / 8 + 2 * (x - pair_units);
+    c1 = c0 + 1;
+    o0 = *(const uint4*)(qh + 8 * c0);
+    o1 = *(const uint4*)(qh + 8 * c1);
+    return;
+  }
+  c0 = x;
+  c1 = x + pair_units;
+  const int i0 = 8 * x;
+  const uint4 ra = *(const uint4*)(qh + i0);
+  const uint4 rb = *(const uint4*)(qh + i0 + rope.half);
+  const uint32_t wa[4] = {ra.x, ra.y, ra.z, ra.w}, wb[4] = {rb.x, rb.y, rb.z, rb.w};
+  uint32_t lo[4], hi[4];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    float y1[2], y2[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const S xa = __builtin_bit_cast(S, (uint16_t)(wa[w] >> (16 * b)));
+      const S xb = __builtin_bit_cast(S, (uint16_t)(wb[w] >> (16 * b)));
+      float cs, sn;
+      rope_cos_sin(rope, p, i0 + 2 * w + b, cs, sn);
+      rope_pair<E>(rope, cs, sn, E::load(xa), E::load(xb), y1[b], y2[b]);
+    }
+    lo[w] = Mma<E>::pack(y1[0], y1[1]);  // already representable: the conversions are exact
+    hi[w] = Mma<E>::pack(y2[0], y2[1]);
+  }
+  o0 = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+  o1 = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+}
+
 // Wait until the matrix pipe has written the results of products issued from assembly
 // (run32_acc): 8 passes plus the write-back, 20 wait states.
 __device__ __forceinline__ void accumulator_fence() { asm volatile("s_nop 15\n\ts_nop 3" ::: "memory"); }

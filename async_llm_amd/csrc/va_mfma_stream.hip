@@ -192,19 +192,20 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
 
     // rotate the query tile into the last buffer (not yet in use), swizzled like a K tile
     va_u32x4* q_stage = ring + (kBuffers - 1) * 2 * kTileUnits;
-    for (int idx = tid; idx < 16 * kChunks; idx += kStreamThreads) {
-      const int jr = idx / kChunks, c = idx - jr * kChunks;
+    for (int idx = tid; idx < 16 * (kChunks / 2); idx += kStreamThreads) {  // two pieces per step
+      const int jr = idx / (kChunks / 2), x = idx - jr * (kChunks / 2);
       const int iq = jr / G, g = jr - iq * G;
-      va_u32x4 packed = {0, 0, 0, 0};
+      int c0 = 2 * x, c1 = 2 * x + 1;
+      uint4 p0 = make_uint4(0, 0, 0, 0), p1 = p0;
       if (iq < n_q) {
         const int subrow = (lflags & VA_LINK_INDIRECT) ? a.qrefs[qref + iq] : qref + iq;
         const long long src_row = a.sub_worker[subrow];
         const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
         const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
-        const uint4 piece = rotated_query_piece<E>(a.rope, qh, c * 8, p);
-        packed = va_u32x4{piece.x, piece.y, piece.z, piece.w};
+        rotated_query_unit<E>(a.rope, qh, x, p, c0, c1, p0, p1);
       }
-      q_stage[jr * kChunks + (c ^ swz<kD>(jr))] = packed;
+      q_stage[jr * kChunks + (c0 ^ swz<kD>(jr))] = va_u32x4{p0.x, p0.y, p0.z, p0.w};
+      q_stage[jr * kChunks + (c1 ^ swz<kD>(jr))] = va_u32x4{p1.x, p1.y, p1.z, p1.w};
     }
     ring_barrier<kAnyInFlight>();
     va_u32x4 qf[kSteps];  // B operands: row j, dims [32s + 8kg, +8)

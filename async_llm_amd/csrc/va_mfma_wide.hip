@@ -209,20 +209,21 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     va_u32x4 qf[kB][kSteps];  // B operands: row of block b, dims [16s + 8h, +8)
 #pragma unroll
     for (int pass = 0; pass < kB; ++pass) {
-      for (int idx = tid; idx < 128 * kChunks; idx += kWideThreads) {
-        const int Rl = idx / kChunks, c = idx - Rl * kChunks;
+      for (int idx = tid; idx < 128 * (kChunks / 2); idx += kWideThreads) {  // two pieces per step
+        const int Rl = idx / (kChunks / 2), x = idx - Rl * (kChunks / 2);
         const int R = kWaveRows * (Rl / 32) + 32 * pass + Rl % 32;  // block `pass` of every wave
         const int iq = R / G, g = R - iq * G;
-        va_u32x4 packed = {0, 0, 0, 0};
+        int c0 = 2 * x, c1 = 2 * x + 1;
+        uint4 p0 = make_uint4(0, 0, 0, 0), p1 = p0;
         if (iq < n_q) {
           const int subrow = (lflags & VA_LINK_INDIRECT) ? a.qrefs[qref + iq] : qref + iq;
           const long long src_row = a.sub_worker[subrow];
           const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
           const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
-          const uint4 piece = rotated_query_piece<E>(a.rope, qh, c * 8, p);
-          packed = va_u32x4{piece.x, piece.y, piece.z, piece.w};
+          rotated_query_unit<E>(a.rope, qh, x, p, c0, c1, p0, p1);
         }
-        q_stage[Rl * kChunks + (c ^ wide_swz<kD>(Rl))] = packed;
+        q_stage[Rl * kChunks + (c0 ^ wide_swz<kD>(Rl))] = va_u32x4{p0.x, p0.y, p0.z, p0.w};
+        q_stage[Rl * kChunks + (c1 ^ wide_swz<kD>(Rl))] = va_u32x4{p1.x, p1.y, p1.z, p1.w};
       }
       ring_barrier<kAnyInFlight>();
       {
