@@ -366,11 +366,15 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         float sum[kB];
 #pragma unroll
         for (int b = 0; b < kB; ++b) sum[b] = 0.f;
+        // Piece r: the exponential of element r; the sum takes element r - 1 (an exponential's result
+        // is not ready for the very next instruction) and odd pieces pack the finished pair into P.
+        uint32_t pw[kB][8];
         auto exp_piece = [&](int r) __attribute__((always_inline)) {
 #pragma unroll
           for (int b = 0; b < kB; ++b) {
             sc[b][r] = __builtin_amdgcn_exp2f(fmaf(sc[b][r], a.scale_log2, -m_ref[b]));
-            sum[b] += sc[b][r];
+            if (r > 0) sum[b] += sc[b][r - 1];
+            if (r >= 2 && r % 2 == 0) pw[b][r / 2 - 1] = Mma<E>::pack(sc[b][r - 2], sc[b][r - 1]);
           }
         };
         constexpr int kPiecesPerStep = 16 / kSteps > 0 ? 16 / kSteps : 1;  // exponentials between two score steps
@@ -391,7 +395,10 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
           for (int r = 0; r < 16; ++r) exp_piece(r);
         }
 #pragma unroll
-        for (int b = 0; b < kB; ++b) l_run[b] += sum[b];
+        for (int b = 0; b < kB; ++b) {
+          l_run[b] += sum[b] + sc[b][15];
+          pw[b][7] = Mma<E>::pack(sc[b][14], sc[b][15]);
+        }
 
         // ---- phase B: O^T += V^T . P^T over two 16-token steps; while a product runs, the V
         // fragment of the next one is transposed; a transposed fragment serves all row blocks ----
@@ -401,8 +408,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
           for (int b = 0; b < kB; ++b)
-            pf[kk][b] = va_u32x4{Mma<E>::pack(sc[b][8 * kk + 0], sc[b][8 * kk + 1]), Mma<E>::pack(sc[b][8 * kk + 2], sc[b][8 * kk + 3]),
-                                 Mma<E>::pack(sc[b][8 * kk + 4], sc[b][8 * kk + 5]), Mma<E>::pack(sc[b][8 * kk + 6], sc[b][8 * kk + 7])};
+            pf[kk][b] = va_u32x4{pw[b][4 * kk + 0], pw[b][4 * kk + 1], pw[b][4 * kk + 2], pw[b][4 * kk + 3]};
         auto transposed = [&](int idx) __attribute__((always_inline)) {
           const int kk = idx / kDimTiles, t = idx % kDimTiles;
           const int w = t / 2;
