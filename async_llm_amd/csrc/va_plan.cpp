@@ -97,7 +97,10 @@ inline int32_t visible_end(int32_t len, int32_t nq, bool causal, int32_t b) {
   return causal ? std::min(len, len - nq + b) : len;
 }
 
-int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* params, Built& out) {
+// `cap`, when given, bounds the number of entries a die may receive in each class, so that a plan
+// whose real items fit the capacity still fits it after the per-die padding.
+int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* params, Built& out,
+          const VaPlanCapacity* cap = nullptr) {
   int rc = check_subs(s, shape);
   if (rc) return rc;
   const int kernel = resolve_kernel(shape, params);
@@ -416,11 +419,43 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     std::iota(by_cost.begin(), by_cost.end(), 0);
     std::stable_sort(by_cost.begin(), by_cost.end(), [&](int32_t x, int32_t y) { return units[x].cost > units[y].cost; });
     int64_t load[kXcds] = {0};
+    int64_t room[kXcds];
+    std::fill(room, room + kXcds, cap ? (kind ? cap->max_wide_items : cap->max_items) / kXcds : INT32_MAX);
     std::vector<int32_t> die_units[kXcds];
-    for (int32_t u : by_cost) {
-      const int die = (int)(std::min_element(load, load + kXcds) - load);
+    // least loaded die that still has room for `n` entries (-1: none)
+    auto pick_die = [&](int64_t n) {
+      int best = -1;
+      for (int d = 0; d < kXcds; ++d)
+        if (room[d] >= n && (best < 0 || load[d] < load[best])) best = d;
+      return best;
+    };
+    auto place = [&](int32_t u, int die) {
       die_units[die].push_back(u);
       load[die] += units[u].cost;
+      room[die] -= (int64_t)units[u].members.size();
+    };
+    for (size_t k = 0; k < by_cost.size(); ++k) {
+      const int32_t u = by_cost[k];
+      int die = pick_die((int64_t)units[u].members.size());
+      if (die >= 0) {
+        place(u, die);
+        continue;
+      }
+      // No die has room for the whole unit (fixed capacity only): its tiles go one by one to dies
+      // that have room, at the price of fetching the chunk once per die.  When even that fails the
+      // plan is over capacity, which the serializer reports; keep every item in the launch order.
+      const std::vector<int32_t> members = units[u].members;
+      units[u].members.clear();
+      units[u].cost = units[u].item_cost = 0;
+      for (int32_t m : members) {
+        Unit single;
+        single.cost = single.item_cost = out.items[m].tokens;
+        single.members.push_back(m);
+        units.push_back(single);
+        die = pick_die(1);
+        if (die < 0) die = (int)(std::min_element(load, load + kXcds) - load);
+        place((int32_t)units.size() - 1, die);
+      }
     }
     std::vector<int32_t> die_items[kXcds];
     size_t depth = 0;
@@ -483,70 +518,200 @@ extern "C" int va_plan_count(const VaSubRequests* subs, const VaShape* shape, co
   return VA_OK;
 }
 
-extern "C" int va_plan_build(const VaSubRequests* subs, const VaShape* shape, const VaPlanParams* params,
-                             int32_t* plan_host, int64_t plan_capacity_words, VaPlanCounts* counts) {
-  if (!plan_host) return va_fail(VA_ERR_ARG, "null plan buffer");
-  Built b;
-  int rc = build(subs, shape, params, b);
-  if (rc) return rc;
+// Serialise a built plan.  With `cap` the sections sit at offsets that depend on the capacity
+// alone and the item lists are padded to it; otherwise they are packed.
+static int write_plan(const Built& b, const VaSubRequests* subs, const VaShape* shape, const VaPlanCapacity* cap,
+                      int32_t* plan_host, int64_t plan_capacity_words, VaPlanCounts* counts) {
   VaPlanCounts c;
   fill_counts(b, subs, shape, &c);
+  const int32_t n_narrow = c.n_items - c.n_wide_items;
+  int32_t cap_wide = c.n_wide_items, cap_narrow = n_narrow, cap_links = c.n_links, cap_qrefs = c.n_qrefs,
+          cap_row_parts = c.n_row_parts, cap_rows = subs->n_rows, cap_partials = c.n_partials;
+  if (cap) {
+    if (cap->max_items % 8 || cap->max_wide_items % 8 || cap->max_items < 0 || cap->max_wide_items < 0)
+      return va_fail(VA_ERR_ARG, "capacity: item counts must be non-negative multiples of 8");
+#define VA_FITS(have, room, what) \
+  if ((have) > (room)) return va_fail(VA_ERR_CAPACITY, "plan exceeds the fixed capacity: %d %s, room for %d", (have), what, (room));
+    VA_FITS(c.n_wide_items, cap->max_wide_items, "wide work items")
+    VA_FITS(n_narrow, cap->max_items, "work items")
+    VA_FITS(c.n_links, cap->max_links, "links")
+    VA_FITS(c.n_qrefs, cap->max_qrefs, "query references")
+    VA_FITS(c.n_partials, cap->max_partials, "partial states")
+    VA_FITS(c.n_row_parts, cap->max_row_parts, "row parts")
+    VA_FITS(subs->n_rows, cap->max_rows, "rows")
+#undef VA_FITS
+    cap_wide = cap->max_wide_items; cap_narrow = cap->max_items; cap_links = cap->max_links; cap_qrefs = cap->max_qrefs;
+    cap_row_parts = cap->max_row_parts; cap_rows = cap->max_rows; cap_partials = cap->max_partials;
+    c.n_items = cap_wide + cap_narrow;
+    c.n_wide_items = cap_wide;
+    c.n_links = cap_links;
+    c.n_qrefs = cap_qrefs;
+    c.n_partials = cap_partials;
+    c.n_row_parts = cap_row_parts;
+    c.plan_words = (int32_t)va_plan_fixed_words(cap);
+    c.workspace_bytes = va_workspace_bytes_for(cap_partials, shape->num_q_heads, shape->head_dim);
+  }
   if (plan_capacity_words < c.plan_words)
     return va_fail(VA_ERR_CAPACITY, "plan needs %d words, buffer holds %lld", c.plan_words,
                    (long long)plan_capacity_words);
   int32_t* h = plan_host;
+  std::memset(h, 0, sizeof(int32_t) * (size_t)c.plan_words);
   int32_t off = VA_PLAN_HEADER_WORDS;
-  std::memset(h, 0, sizeof(int32_t) * VA_PLAN_HEADER_WORDS);
   h[VA_H_MAGIC] = VA_PLAN_MAGIC;
   h[VA_H_KERNEL] = c.kernel;
   h[VA_H_Q_TILE] = c.q_tile;
-  h[VA_H_KV_CHUNK] = c.kv_chunk;
-  h[VA_H_N_WIDE] = c.n_wide_items;
+  h[VA_H_KV_CHUNK] = cap ? 0 : c.kv_chunk;  // chosen per plan: not part of a fixed plan's header (see counts)
+  h[VA_H_N_WIDE] = cap_wide;
   h[VA_H_WIDE_TILE] = c.wide_tile;
-  h[VA_H_N_ITEMS] = c.n_items;
-  h[VA_H_N_LINKS] = c.n_links;
-  h[VA_H_N_QREFS] = c.n_qrefs;
-  h[VA_H_N_PARTIALS] = c.n_partials;
-  h[VA_H_N_ROW_PARTS] = c.n_row_parts;
-  h[VA_H_N_ROWS] = subs->n_rows;
-  h[VA_H_N_SUBROWS] = subs->n_subrows;
-  h[VA_H_N_EMPTY_ROWS] = (int32_t)std::count(b.row_flags.begin(), b.row_flags.end(), VA_ROW_EMPTY);
+  h[VA_H_N_ITEMS] = cap_wide + cap_narrow;
+  h[VA_H_N_LINKS] = cap_links;
+  h[VA_H_N_QREFS] = cap_qrefs;
+  h[VA_H_N_PARTIALS] = cap_partials;
+  h[VA_H_N_ROW_PARTS] = cap_row_parts;
+  h[VA_H_N_ROWS] = cap_rows;
+  // a fixed plan's header depends on the capacity alone: these two words hold their upper bounds
+  h[VA_H_N_SUBROWS] = cap ? cap_qrefs : subs->n_subrows;
+  h[VA_H_N_EMPTY_ROWS] = cap ? cap_rows : (int32_t)std::count(b.row_flags.begin(), b.row_flags.end(), VA_ROW_EMPTY);
   h[VA_H_OFF_ITEMS] = off;
-  for (auto& it : b.items) {
-    int32_t* w = plan_host + off;
-    std::memset(w, 0, sizeof(int32_t) * VA_ITEM_WORDS);
+  auto write_item = [&](int32_t at, const Item& it) {
+    int32_t* w = plan_host + off + at * VA_ITEM_WORDS;
     w[VA_I_LINK_BEGIN] = it.link_begin;
     w[VA_I_N_LINKS] = it.n_links;
     w[VA_I_N_Q] = it.n_q;
     w[VA_I_PART_BASE] = it.part_base;
     w[VA_I_TOKENS] = it.tokens;
     w[VA_I_KIND] = it.kind;
-    off += VA_ITEM_WORDS;
-  }
+  };
+  for (int32_t i = 0; i < b.n_wide; ++i) write_item(i, b.items[i]);
+  for (int32_t i = b.n_wide; i < cap_wide; ++i) write_item(i, Item{0, 0, 0, -1, 0, 1, -1});
+  for (int32_t i = 0; i < n_narrow; ++i) write_item(cap_wide + i, b.items[b.n_wide + i]);
+  for (int32_t i = n_narrow; i < cap_narrow; ++i) write_item(cap_wide + i, Item{0, 0, 0, -1, 0, 0, -1});
+  off += (cap_wide + cap_narrow) * VA_ITEM_WORDS;
   h[VA_H_OFF_LINKS] = off;
-  for (auto& l : b.links) {
-    int32_t* w = plan_host + off;
-    std::memset(w, 0, sizeof(int32_t) * VA_LINK_WORDS);
+  for (size_t i = 0; i < b.links.size(); ++i) {
+    const Link& l = b.links[i];
+    int32_t* w = plan_host + off + (int32_t)i * VA_LINK_WORDS;
     w[VA_L_KV_BEGIN] = l.kv_begin;
     w[VA_L_TOK_BEGIN] = l.tok_begin;
     w[VA_L_TOK_END] = l.tok_end;
     w[VA_L_QREF] = l.qref;
     w[VA_L_CAUSAL_BASE] = l.causal_base;
     w[VA_L_FLAGS] = l.flags;
-    off += VA_LINK_WORDS;
   }
+  off += cap_links * VA_LINK_WORDS;
   h[VA_H_OFF_QREFS] = off;
   std::copy(b.qrefs.begin(), b.qrefs.end(), plan_host + off);
-  off += c.n_qrefs;
+  off += cap_qrefs;
   h[VA_H_OFF_ROW_INDPTR] = off;
   std::copy(b.row_indptr.begin(), b.row_indptr.end(), plan_host + off);
-  off += subs->n_rows + 1;
+  for (int32_t r = subs->n_rows; r < cap_rows; ++r) plan_host[off + r + 1] = b.row_indptr.back();
+  off += cap_rows + 1;
   h[VA_H_OFF_ROW_IDS] = off;
   std::copy(b.row_ids.begin(), b.row_ids.end(), plan_host + off);
-  off += c.n_row_parts;
+  off += cap_row_parts;
   h[VA_H_OFF_ROW_FLAGS] = off;
   std::copy(b.row_flags.begin(), b.row_flags.end(), plan_host + off);
-  off += subs->n_rows;
+  for (int32_t r = subs->n_rows; r < cap_rows; ++r) plan_host[off + r] = VA_ROW_EMPTY;
+  off += cap_rows;
   if (counts) *counts = c;
   return VA_OK;
+}
+
+extern "C" int va_plan_build(const VaSubRequests* subs, const VaShape* shape, const VaPlanParams* params,
+                             int32_t* plan_host, int64_t plan_capacity_words, VaPlanCounts* counts) {
+  if (!plan_host) return va_fail(VA_ERR_ARG, "null plan buffer");
+  Built b;
+  int rc = build(subs, shape, params, b);
+  if (rc) return rc;
+  return write_plan(b, subs, shape, nullptr, plan_host, plan_capacity_words, counts);
+}
+
+extern "C" int64_t va_plan_fixed_words(const VaPlanCapacity* cap) {
+  if (!cap) return 0;
+  return (int64_t)VA_PLAN_HEADER_WORDS + ((int64_t)cap->max_items + cap->max_wide_items) * VA_ITEM_WORDS +
+         (int64_t)cap->max_links * VA_LINK_WORDS + cap->max_qrefs + (cap->max_rows + 1) + cap->max_row_parts +
+         cap->max_rows;
+}
+
+// Upper bounds of every plan section for a workload within `lim`, following the rules of build():
+//   * stand-alone sub-requests: a group of readers is cut into tiles x chunks with
+//     chunk >= total_tokens / target, so items <= tiles + target with tiles <= sub-requests; every
+//     item carries one link; a query row enters the partial list once per chunk of its run;
+//   * chains: tiles of up to wide_tile rows (the last one of a chain may be narrow), each split
+//     into at most ceil(target / tiles) pieces, so items <= tiles + target per class; a tile has
+//     one link per member plus one per cut; a split tile's rows enter the partial list once per piece.
+extern "C" int va_plan_capacity(const VaShape* shape, const VaPlanParams* params, const VaPlanLimits* lim,
+                                VaPlanCapacity* capacity) {
+  if (!shape || !lim || !capacity) return va_fail(VA_ERR_ARG, "null argument");
+  if (params && params->kv_chunk > 0)
+    return va_fail(VA_ERR_ARG, "fixed-capacity plans choose their KV chunk themselves: kv_chunk must be 0");
+  if (lim->max_sub_requests < 0 || lim->max_sub_rows < lim->max_sub_requests || lim->max_chains < 0 ||
+      lim->max_chain_members < 0 || lim->max_chain_rows < 0 || lim->max_rows <= 0)
+    return va_fail(VA_ERR_ARG, "limits: negative count, no rows, or fewer query rows than sub-requests");
+  if (shape->num_kv_heads <= 0 || shape->num_q_heads % shape->num_kv_heads)
+    return va_fail(VA_ERR_ARG, "num_q_heads must be a multiple of num_kv_heads");
+  const int kernel = resolve_kernel(shape, params);
+  if (kernel < 0) return va_fail(VA_ERR_ARG, "requested kernel family does not support this dtype/shape");
+  const int g = shape->num_q_heads / shape->num_kv_heads;
+  const int64_t q_tile = params && params->q_tile > 0 ? params->q_tile
+                                                      : (kernel == VA_KERNEL_MFMA ? va_mfma_default_q_tile(g, false) : 1);
+  int64_t wide_tile = 0;
+  if (kernel == VA_KERNEL_MFMA && !(params && params->wide_tile < 0)) {
+    wide_tile = params && params->wide_tile > 0 ? params->wide_tile : va_mfma_wide_q_tile(g, shape->head_dim);
+    if (wide_tile <= q_tile) wide_tile = 0;
+  }
+  const bool wide_groups = params && params->wide_tile > 0 && wide_tile > 0;
+  const int64_t target = params && params->target_items > 0 ? params->target_items
+                                                            : std::max(64, 2048 / shape->num_kv_heads);
+  const int64_t subs = lim->max_sub_requests, sub_rows = lim->max_sub_rows;
+  const int64_t chains = lim->max_chains, members = lim->max_chain_members, chain_rows = lim->max_chain_rows;
+
+  int64_t narrow = 0, wide = 0, links = 0, qrefs = 0, partials = 0;
+  if (subs > 0) {
+    narrow += sub_rows + target;  // tiles <= query rows
+    // wide decode tiles are cut at min(chunk, their tokens / (256 / kv heads))
+    if (wide_groups) wide += sub_rows + target + 256;
+    qrefs += sub_rows;
+    // a query row is in one tile; that tile has at most 1 + len / chunk chunks, and the sum of
+    // len / chunk over tiles is at most target (times the tile's rows when counted per row)
+    partials += sub_rows + (q_tile + (wide_groups ? wide_tile : 0)) * (target + 256);
+  }
+  if (chains > 0 && chain_rows > 0) {
+    const int64_t tile_rows = wide_tile ? wide_tile : q_tile;
+    const int64_t tiles = chain_rows / tile_rows + chains;  // per chain: floor(rows / tile) + 1
+    if (wide_tile) {
+      wide += tiles + target;
+      narrow += chains + target;
+    } else {
+      narrow += tiles + target;
+    }
+    const int64_t chain_items = tiles + target + (wide_tile ? chains + target : 0);
+    links += tiles * members + chain_items;
+    partials += chain_rows + tile_rows * target;
+  }
+  links += narrow + wide;
+  auto round8 = [](int64_t x) { return (x + 7) / 8 * 8; };
+  const int64_t limit = INT32_MAX / 64;
+  if (narrow > limit || wide > limit || links > limit || partials > limit)
+    return va_fail(VA_ERR_CAPACITY, "limits describe a plan too large for 32-bit tables");
+  capacity->max_items = (int32_t)round8(narrow);
+  capacity->max_wide_items = (int32_t)round8(wide);
+  capacity->max_links = (int32_t)links;
+  capacity->max_qrefs = (int32_t)qrefs;
+  capacity->max_partials = (int32_t)partials;
+  capacity->max_row_parts = (int32_t)partials;
+  capacity->max_rows = lim->max_rows;
+  return VA_OK;
+}
+
+extern "C" int va_plan_build_fixed(const VaSubRequests* subs, const VaShape* shape, const VaPlanParams* params,
+                                   const VaPlanCapacity* cap, int32_t* plan_host, int64_t plan_capacity_words,
+                                   VaPlanCounts* counts) {
+  if (!plan_host || !cap) return va_fail(VA_ERR_ARG, "null plan buffer or capacity");
+  if (cap->max_items % kXcds || cap->max_wide_items % kXcds || cap->max_items < 0 || cap->max_wide_items < 0)
+    return va_fail(VA_ERR_ARG, "capacity: item counts must be non-negative multiples of 8");
+  Built b;
+  int rc = build(subs, shape, params, b, cap);
+  if (rc) return rc;
+  return write_plan(b, subs, shape, cap, plan_host, plan_capacity_words, counts);
 }

@@ -21,6 +21,7 @@ VA_ROPE_TABLE, VA_ROPE_MROPE = 0, 1
 VA_KERNEL_AUTO, VA_KERNEL_GENERIC, VA_KERNEL_MFMA = 0, 1, 2
 VA_SUB_CAUSAL, VA_SUB_SLOTS = 1, 2
 PLAN_HEADER_WORDS = 24
+VA_ERR_ARG, VA_ERR_CAPACITY = -1, -2
 
 _DTYPES = {torch.float32: VA_F32, torch.float16: VA_F16, torch.bfloat16: VA_BF16}
 
@@ -31,6 +32,9 @@ EXPORTED_SYMBOLS = (
     "va_store_kv_rope",
     "va_plan_count",
     "va_plan_build",
+    "va_plan_capacity",
+    "va_plan_fixed_words",
+    "va_plan_build_fixed",
     "va_attention",
 )
 
@@ -99,6 +103,23 @@ class VaPlanCounts(C.Structure):
     ]
 
 
+class VaPlanLimits(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("max_sub_requests", "max_sub_rows", "max_chains", "max_chain_members",
+                                         "max_chain_rows", "max_rows")]
+
+
+class VaPlanCapacity(C.Structure):
+    _fields_ = [
+        ("max_items", C.c_int32),
+        ("max_wide_items", C.c_int32),
+        ("max_links", C.c_int32),
+        ("max_qrefs", C.c_int32),
+        ("max_partials", C.c_int32),
+        ("max_row_parts", C.c_int32),
+        ("max_rows", C.c_int32),
+    ]
+
+
 def _load() -> C.CDLL:
     if not os.path.exists(LIB_PATH):
         raise ImportError(
@@ -117,6 +138,14 @@ def _load() -> C.CDLL:
     lib.va_plan_count.restype = C.c_int
     lib.va_plan_count.argtypes = [C.POINTER(VaSubRequests), C.POINTER(VaShape), C.POINTER(VaPlanParams),
                                   C.POINTER(VaPlanCounts)]
+    lib.va_plan_capacity.restype = C.c_int
+    lib.va_plan_capacity.argtypes = [C.POINTER(VaShape), C.POINTER(VaPlanParams), C.POINTER(VaPlanLimits),
+                                     C.POINTER(VaPlanCapacity)]
+    lib.va_plan_fixed_words.restype = C.c_int64
+    lib.va_plan_fixed_words.argtypes = [C.POINTER(VaPlanCapacity)]
+    lib.va_plan_build_fixed.restype = C.c_int
+    lib.va_plan_build_fixed.argtypes = [C.POINTER(VaSubRequests), C.POINTER(VaShape), C.POINTER(VaPlanParams),
+                                        C.POINTER(VaPlanCapacity), C.c_void_p, C.c_int64, C.POINTER(VaPlanCounts)]
     lib.va_plan_build.restype = C.c_int
     lib.va_plan_build.argtypes = [C.POINTER(VaSubRequests), C.POINTER(VaShape), C.POINTER(VaPlanParams),
                                   vp, i64, C.POINTER(VaPlanCounts)]

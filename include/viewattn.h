@@ -177,6 +177,64 @@ VA_API int va_plan_build(const VaSubRequests* subs, const VaShape* shape, const 
                   int32_t* plan_host, int64_t plan_capacity_words, VaPlanCounts* counts);
 
 /*
+ * Fixed-capacity plans, for launches that are recorded once and replayed (HIP
+ * graphs): the reference keeps such plans in fixed slot geometry
+ * (shared_cache/attention_graph.py:14-121 decode, :127-290 prefill; workspace
+ * sizing attention.py:212-239).  Here the geometry that must not change between
+ * replays is what va_attention derives from the plan header: the number of
+ * workgroups of each launch, the merge grid and the section offsets.
+ * va_plan_build_fixed lays the sections out at offsets given by `capacity` alone
+ * and pads the item lists with empty items, so every plan built with the same
+ * capacity has the same header and va_attention issues the same launches on the
+ * same buffers; only the contents of the plan blob (and of kv_indices,
+ * sub_worker, sub_loc) change.  (Three informational header words differ from a packed
+ * plan's: the sub-row and empty-row counts hold max_qrefs and max_rows, and the
+ * KV chunk, which is chosen per plan, reads 0; counts->kv_chunk has it.)  Rows beyond subs->n_rows, up to max_rows, get
+ * out = 0 and lse = -inf.  A plan that does not fit returns VA_ERR_CAPACITY and
+ * names the section.
+ */
+typedef struct VaPlanCapacity {
+  int32_t max_items;       /* narrow work items, a multiple of 8            */
+  int32_t max_wide_items;  /* wide work items, a multiple of 8 (may be 0)   */
+  int32_t max_links;
+  int32_t max_qrefs;
+  int32_t max_partials;    /* sizes the workspace                           */
+  int32_t max_row_parts;
+  int32_t max_rows;        /* rows of `out` the launch covers               */
+} VaPlanCapacity;
+
+/*
+ * What a fixed-capacity launch must be able to hold, in the planner's own terms.
+ * The reference sizes its graph buffers from (workers, depth, max_pages) for decode
+ * (attention_graph.py:15-31) and (workers, depth, rows, max_pages) for prefill
+ * (attention_graph.py:137-163):
+ *   decode : max_sub_requests = max_sub_rows = workers * (depth + 1), max_rows = workers
+ *   prefill: max_chains = workers, max_chain_members = depth + 1, max_chain_rows = rows,
+ *            max_rows = rows
+ * va_plan_capacity turns them into section sizes that no plan within the limits can
+ * exceed (the KV chunk is chosen per plan, so page counts do not enter; kv_indices is
+ * the caller's buffer).  params->kv_chunk must be 0.
+ */
+typedef struct VaPlanLimits {
+  int32_t max_sub_requests;   /* stand-alone (decode) sub-requests, empty ones included */
+  int32_t max_sub_rows;       /* their query rows in total                               */
+  int32_t max_chains;         /* prefill requests                                        */
+  int32_t max_chain_members;  /* sub-requests per prefill request                        */
+  int32_t max_chain_rows;     /* new tokens of all prefill requests together             */
+  int32_t max_rows;           /* rows of `out`                                           */
+} VaPlanLimits;
+
+VA_API int va_plan_capacity(const VaShape* shape, const VaPlanParams* params, const VaPlanLimits* limits,
+                     VaPlanCapacity* capacity);
+
+/* int32 words of a fixed-capacity plan blob */
+VA_API int64_t va_plan_fixed_words(const VaPlanCapacity* capacity);
+
+VA_API int va_plan_build_fixed(const VaSubRequests* subs, const VaShape* shape, const VaPlanParams* params,
+                        const VaPlanCapacity* capacity, int32_t* plan_host, int64_t plan_capacity_words,
+                        VaPlanCounts* counts);
+
+/*
  * va_attention: out[r, h, :] = softmax over the whole view of row r, i.e. the
  * LSE merge over all sub-requests (and KV chunks) that serve row r of
  *   softmax(R(sub_loc[i]) q[sub_worker[i], h] . K_s^T / sqrt(head_dim)) V_s .

@@ -128,17 +128,11 @@ def run_decode_parity(op, cpu_pool, dev_pool, group, page_alloc, theta, gen, sca
     return out, lse, exp_out, exp_lse, meta
 
 
-def run_prefill_parity(op, cpu_pool, dev_pool, specs, theta, gen, scale=None):
-    """One batched prefill through the product op and through the oracle."""
-    from types import SimpleNamespace
-
-    dev = op.device
+def prefill_inputs(op, specs, gen, scale=None):
+    """Write positions, destination slots and random q/k/v rows (CPU tensors) of a
+    batched prefill, request-major: ``(positions, mrope_positions, out_loc, q, k, v)``."""
     Hq, Hkv, D, P = op.num_qo_heads, op.num_kv_heads, op.head_dim, op.page_size
     scale = D ** -0.5 if scale is None else scale
-    meta = op.prepare_prefill_batch(specs)
-    oplan = oracle_prefill_plan(specs, P)
-    assert torch.equal(meta.sub_loc.cpu(), oplan.sub_loc) and meta.pad_slot.tolist() == oplan.pad_slot
-    N = meta.num_workers
     use_3d = any(s.mrope_rel is not None for s in specs) or op.mrope_section is not None
     positions, mpos, out_loc = [], [], []
     for s in specs:
@@ -153,25 +147,48 @@ def run_prefill_parity(op, cpu_pool, dev_pool, specs, theta, gen, scale=None):
     positions = torch.cat(positions)
     mrope_positions = torch.cat(mpos, dim=1) if use_3d else None
     out_loc = torch.cat(out_loc)
+    N = positions.numel()
     q = (torch.randn(N, Hq * D, generator=gen) * scale).to(op.dtype)
     k = (torch.randn(N, Hkv * D, generator=gen) * scale).to(op.dtype)
     v = (torch.randn(N, Hkv * D, generator=gen) * scale).to(op.dtype)
-    batch = SimpleNamespace(attn_metadata=meta, positions=positions.to(dev), out_loc=out_loc.to(dev),
-                            mrope_positions=None if mrope_positions is None else mrope_positions.to(dev))
-    out, lse = op.forward_with_lse(q.to(dev), k.to(dev), v.to(dev), 0, batch)
-    torch.cuda.synchronize()
+    return positions, mrope_positions, out_loc, q, k, v
 
+
+def oracle_prefill(op, cpu_pool, specs, theta, positions, mrope_positions, out_loc, q, k, v):
+    """Store the new rows into the CPU pool and run the oracle's batched prefill."""
+    Hq, Hkv, D, P = op.num_qo_heads, op.num_kv_heads, op.head_dim, op.page_size
+    N = q.shape[0]
     rope = oracle_rope(op, theta)
     k_cpu, v_cpu = cpu_pool
     key_pos = positions if mrope_positions is None else mrope_positions
     k_rot = rope.rotate(k.view(N, Hkv, D), key_pos)
     O.store_kv(k_cpu.view(-1, Hkv * D), v_cpu.view(-1, Hkv * D), out_loc, k_rot.reshape(N, -1), v)
+    return O.forward_prefill_batch(oracle_prefill_plan(specs, P), q.view(N, Hq, D), k_cpu, v_cpu, rope)
+
+
+def run_prefill_parity(op, cpu_pool, dev_pool, specs, theta, gen, scale=None):
+    """One batched prefill through the product op and through the oracle."""
+    from types import SimpleNamespace
+
+    dev = op.device
+    Hq, D, P = op.num_qo_heads, op.head_dim, op.page_size
+    meta = op.prepare_prefill_batch(specs)
+    oplan = oracle_prefill_plan(specs, P)
+    assert torch.equal(meta.sub_loc.cpu(), oplan.sub_loc) and meta.pad_slot.tolist() == oplan.pad_slot
+    N = meta.num_workers
+    positions, mrope_positions, out_loc, q, k, v = prefill_inputs(op, specs, gen, scale)
+    batch = SimpleNamespace(attn_metadata=meta, positions=positions.to(dev), out_loc=out_loc.to(dev),
+                            mrope_positions=None if mrope_positions is None else mrope_positions.to(dev))
+    out, lse = op.forward_with_lse(q.to(dev), k.to(dev), v.to(dev), 0, batch)
+    torch.cuda.synchronize()
+
+    exp_out, exp_lse = oracle_prefill(op, cpu_pool, specs, theta, positions, mrope_positions, out_loc, q, k, v)
+    k_cpu, v_cpu = cpu_pool
     assert torch.equal(dev_pool[1].cpu(), v_cpu), "V pool differs"
     if op.mrope_section is None:
         assert torch.equal(dev_pool[0].cpu(), k_cpu), "K pool differs"
     else:
         assert_close(dev_pool[0].cpu().float(), k_cpu.float(), op.dtype, "K pool")
-    exp_out, exp_lse = O.forward_prefill_batch(oplan, q.view(N, Hq, D), k_cpu, v_cpu, rope)
     assert out.shape == (N, Hq * D)
     assert_close(out, exp_out, op.dtype, "out")
     assert_close(lse, exp_lse, op.dtype, "lse")
