@@ -12,7 +12,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libviewattn.so")
-SOURCES = ["viewattn.hip", "va_mfma.hip", "va_mfma_wide.hip", "va_mfma_stream.hip", "va_plan.cpp"]
+SOURCES = ["viewattn.hip", "va_mfma.hip", "va_mfma_wide.hip", "va_mfma_stream.hip", "va_block_copy.hip", "va_plan.cpp"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -42,6 +42,9 @@ struct MergeArgs {
   int num_q_heads, head_dim;
 };
 
+// Validate a rotation description and turn it into its device form.
+int make_rope(const VaRope* rope, int head_dim, RopeDev* out);
+
 // Matrix-core attention (launched from va_mfma.hip).
 // `n_wide` leading items are wide tiles (va_mfma_wide.hip), the rest narrow ones (va_mfma_stream.hip).
 int launch_mfma(const AttnArgs& a, int dtype, int n_items, int n_wide, int q_tile, hipStream_t stream);

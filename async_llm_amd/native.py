@@ -32,6 +32,7 @@ EXPORTED_SYMBOLS = (
     "va_store_kv_rope",
     "va_plan_count",
     "va_plan_build",
+    "va_copy_shift_kv",
     "va_plan_capacity",
     "va_plan_fixed_words",
     "va_plan_build_fixed",
@@ -135,6 +136,8 @@ def _load() -> C.CDLL:
     lib.va_store_kv_rope.restype = C.c_int
     lib.va_store_kv_rope.argtypes = [vp, vp, i64, i64, vp, vp, i64, vp, i32, vp, i64, i64,
                                      C.POINTER(VaShape), C.POINTER(VaRope), vp]
+    lib.va_copy_shift_kv.restype = C.c_int
+    lib.va_copy_shift_kv.argtypes = [vp, vp, i64, i64, i32, vp, vp, i64, i64, C.POINTER(VaShape), C.POINTER(VaRope), vp]
     lib.va_plan_count.restype = C.c_int
     lib.va_plan_count.argtypes = [C.POINTER(VaSubRequests), C.POINTER(VaShape), C.POINTER(VaPlanParams),
                                   C.POINTER(VaPlanCounts)]

@@ -16,6 +16,11 @@
  *   attention.py:652-703 (q gather + per-segment rotate,    va_attention
  *     BatchDecode run x2, pad-scatter, merge_states) and
  *     attention.py:705-752 (BatchPrefill run x2, merge)
+ *   attention_graph.py:14-290 (fixed-capacity graph        va_plan_capacity,
+ *     buffers) + attention.py:212-239 (workspace sizing)    va_plan_fixed_words,
+ *                                                           va_plan_build_fixed
+ *   session.py:470-528 (block merge / append: KV copy and   va_copy_shift_kv
+ *     key shift into the left block's position frame)
  *
  * Conventions: every function returns 0 on success or a negative VA_ERR_*;
  * va_last_error() returns a thread-local message for the last failure.  All
@@ -233,6 +238,27 @@ VA_API int64_t va_plan_fixed_words(const VaPlanCapacity* capacity);
 VA_API int va_plan_build_fixed(const VaSubRequests* subs, const VaShape* shape, const VaPlanParams* params,
                         const VaPlanCapacity* capacity, int32_t* plan_host, int64_t plan_capacity_words,
                         VaPlanCounts* counts);
+
+/*
+ * va_copy_shift_kv: block merge / append.  For every layer l < num_layers and
+ * token i < n_tokens
+ *   k_pool_l[dst[i]] = round(R(position_shift) float(k_pool_l[src[i]]))
+ *   v_pool_l[dst[i]] = v_pool_l[src[i]]
+ * where layer l's pools start l * layer_stride ELEMENTS after k_pool_dev /
+ * v_pool_dev (num_layers = 1 for pools that are separate allocations), slots are
+ * int64 on the device and the rotation uses position_shift on all three mRoPE
+ * axes.  position_shift == 0 is a plain copy (rope may be NULL).  The keys are
+ * rotated as fp32 copies and rounded once, as the reference does.  Source and
+ * destination slots must be disjoint sets: the reference gathers everything
+ * before it scatters, this kernel does not.
+ * Replaces session.py:470-528 (_copy_block, _copy_slots, _shift_keys_): per
+ * layer index_select + index_copy_ of K and V, then gather, fp32 rotation and
+ * scatter of the copied keys.
+ */
+VA_API int va_copy_shift_kv(void* k_pool_dev, void* v_pool_dev, int64_t pool_row_stride, int64_t layer_stride,
+                     int32_t num_layers, const int64_t* src_slots_dev, const int64_t* dst_slots_dev,
+                     int64_t n_tokens, int64_t position_shift, const VaShape* shape, const VaRope* rope,
+                     void* stream);
 
 /*
  * va_attention: out[r, h, :] = softmax over the whole view of row r, i.e. the

@@ -19,6 +19,8 @@ path.  All citations are relative to ``/root/reference/python/minisgl``:
   forward_decode             shared_cache/attention.py:624-703
   forward_prefill_batch      shared_cache/attention.py:705-752
   get_rope_index             models/qwen3_5_mrope.py:19-64
+  copy_shift_kv,             shared_cache/session.py:330-420, 478-528 (merge_blocks, append_block,
+  merge_blocks, append_block   _copy_block, _copy_slots, _shift_keys_)
 
 The reference delegates the attention arithmetic itself to FlashInfer 0.6.17
 (``pyproject.toml:31``; CUDA only, not vendored, not installable here).  Its
@@ -47,6 +49,9 @@ How each function is pinned (tests/test_oracle_*.py):
   merge_states,       and the global invariant: segment-wise + merge == ONE softmax over the
   forward_*           concatenated view with keys at absolute positions (attention.py:9-16);
                       K=0,V=1 => out == 1 (test_attention_workspace.py:121-125)
+  copy_shift_kv,      a merged block read as ONE segment equals the closed-form softmax over
+  merge_blocks,       left + right at absolute positions (a wrong sign or amount of the shift fails
+  append_block        it); append == merge slot for slot; self-append doubles; shift 0 is a copy
 parity unpinned: FlashInfer's internal rounding order and the base (e vs 2) of the LSE it
 returns cannot be observed offline; outputs are base-invariant and ``lse_base2`` selects the
 convention for the logsumexp.
@@ -141,6 +146,23 @@ def store_kv(k_pool: torch.Tensor, v_pool: torch.Tensor, out_loc: torch.Tensor, 
     v_pool[slots] = v[keep]
 
 
+def copy_shift_kv(k_pool: torch.Tensor, v_pool: torch.Tensor, src_slots: Sequence[int], dst_slots: Sequence[int],
+                  position_shift: int, rope: "RopeSpec") -> None:
+    """One layer of a block copy: rows ``src_slots`` of the ``[num_slots, Hkv, D]``
+    pools are gathered and written to ``dst_slots`` (session.py:486-507); then, when
+    the destination frame starts ``position_shift`` earlier, the copied keys are
+    gathered again, rotated by it as fp32 and written back in the pool's dtype
+    (session.py:509-528)."""
+    src = torch.as_tensor(src_slots, dtype=torch.int64)
+    dst = torch.as_tensor(dst_slots, dtype=torch.int64)
+    k_pool.index_copy_(0, dst, k_pool.index_select(0, src))
+    v_pool.index_copy_(0, dst, v_pool.index_select(0, src))
+    if position_shift:
+        corrections = torch.full((dst.numel(),), position_shift, dtype=torch.int64)
+        keys = rope.rotate(k_pool.index_select(0, dst).float(), corrections).to(k_pool.dtype)
+        k_pool.index_copy_(0, dst, keys)
+
+
 # ---------------------------------------------------------------------------
 # blocks and planners
 # ---------------------------------------------------------------------------
@@ -191,6 +213,41 @@ class OBlock:
 
     def token_slots(self) -> List[int]:
         return [self.page_starts[i // self.page_size] + i % self.page_size for i in range(self.num_tokens)]
+
+
+def merge_blocks(layers, left: "OBlock", right: "OBlock", alloc_pages, rope: "RopeSpec") -> "OBlock":
+    """``left + right`` in fresh pages (session.py:330-377).  ``layers`` is a list
+    of ``(k_pool, v_pool)`` flat ``[num_slots, Hkv, D]`` views, one per layer;
+    ``alloc_pages(n)`` returns ``n`` page-start slots."""
+    total = left.num_tokens + right.num_tokens
+    merged = OBlock(left.page_size)
+    merged.page_starts = list(alloc_pages(-(-total // left.page_size)))
+    merged.num_tokens = total
+    slots = merged.token_slots()
+    for k_pool, v_pool in layers:
+        if left.num_tokens:
+            copy_shift_kv(k_pool, v_pool, left.token_slots(), slots[: left.num_tokens], 0, rope)
+        if right.num_tokens:
+            copy_shift_kv(k_pool, v_pool, right.token_slots(), slots[left.num_tokens:], left.mrope_span, rope)
+    span = left.mrope_span + right.mrope_span
+    merged.mrope_span_override = None if span == total else span
+    return merged
+
+
+def append_block(layers, left: "OBlock", right: "OBlock", alloc_pages, rope: "RopeSpec") -> "OBlock":
+    """``left += copy of right`` (session.py:379-420); the source layout and both
+    spans are taken before ``left`` grows, so ``right is left`` doubles the block."""
+    left_tokens, left_span, right_span = left.num_tokens, left.mrope_span, right.mrope_span
+    if right.num_tokens:
+        source = right.token_slots()
+        n = right.num_tokens
+        left.grow_pages(list(alloc_pages(left.pages_needed(n))), n)
+        target = left.token_slots()[left_tokens: left_tokens + n]
+        for k_pool, v_pool in layers:
+            copy_shift_kv(k_pool, v_pool, source, target, left_span, rope)
+    span = left_span + right_span
+    left.mrope_span_override = None if span == left.num_tokens else span
+    return left
 
 
 def page_numbers(block, snapshot: Dict[int, List[int]], extra_page: Optional[int] = None) -> List[int]:
