@@ -22,8 +22,14 @@
 
 namespace va {
 
-constexpr int kCopyTokens = 16;  // tokens per workgroup
-constexpr int kCopyBatch = 4;    // tokens whose loads are in flight together
+#ifndef VA_COPY_TOKENS
+#define VA_COPY_TOKENS 16
+#endif
+#ifndef VA_COPY_BATCH
+#define VA_COPY_BATCH 4
+#endif
+constexpr int kCopyTokens = VA_COPY_TOKENS;  // tokens per workgroup
+constexpr int kCopyBatch = VA_COPY_BATCH;    // tokens whose loads are in flight together
 
 template <typename S, int kVec>
 struct alignas(kVec * sizeof(S) == 16 ? 16 : alignof(S)) Piece {

@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="batched_decode",
                     choices=["batched_decode", "mrope_decode", "view_prefill", "plumbing_decode", "mixed_batch",
-                             "copy_calibration"])
+                             "copy_calibration", "block_merge"])
     ap.add_argument("--layers", type=int, default=4, help="copies of the KV pool rotated over")
     ap.add_argument("--kernel", default=None, choices=[None, "auto", "generic", "mfma"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -178,6 +178,107 @@ def copy_calibration(dev, steps):
     return 0
 
 
+def block_merge(dev, steps, warmup, layers, cpu):
+    """Merge of two 16384-token blocks (16 q / 4 kv heads, head_dim 256, bf16, page 16) over
+    ``layers`` layers: left copied, right copied with its keys rotated by the left span.  One step =
+    the two ``va_copy_shift_kv`` launches of ``BlockKVOps.merge_blocks``; algorithmic bytes =
+    4 * layers * kv_heads * head_dim * 2 B per token (K and V, read and written once)."""
+    import numpy as np
+    import torch
+
+    from async_llm_amd.kvcache.mha_pool import MHAKVCache
+    from async_llm_amd.kvcache.page_allocator import PageAllocator
+    from async_llm_amd.shared_cache import BlockKVOps, SharedCacheAttention
+    from async_llm_amd.shared_cache.block_ops import token_slots
+
+    Hq, Hkv, D, P, n_left, n_right = 16, 4, 256, 16, 16384, 16384
+    num_pages = 4 * (n_left + n_right) // P
+    pool = MHAKVCache(Hkv, layers, D, num_pages, P, torch.bfloat16, dev)
+    pool._kv_buffer.normal_()
+    half = D // 2
+    inv = 1.0 / (1e6 ** (torch.arange(half, dtype=torch.float32) / half))
+    angles = torch.arange(32768, dtype=torch.float32)[:, None] * inv[None, :]
+    table = torch.cat([angles.cos(), angles.sin()], dim=-1).to(dev)
+    att = SharedCacheAttention(pool, table, Hq, Hkv, D, P, torch.bfloat16, dev)
+    allocator = PageAllocator(num_pages, P, dev)
+    allocator._free = allocator._free[torch.randperm(num_pages, device=dev)]  # a pool in use: scattered pages
+    ops = BlockKVOps(pool, att, allocator)
+    left, right = ops.create_block(), ops.create_block()
+    left.grow_pages(allocator.alloc_pages(n_left // P), n_left)
+    right.grow_pages(allocator.alloc_pages(n_right // P), n_right)
+    merged = ops.merge_blocks(left, right)
+    torch.cuda.synchronize()
+    src_l, src_r, dst = token_slots(left), token_slots(right), token_slots(merged)
+
+    def step():
+        ops._launch(src_l, dst[:n_left], 0)
+        ops._launch(src_r, dst[n_left:], left.mrope_span)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+    # the launches alone: slot tables already on the device
+    tables = torch.from_numpy(np.stack([np.concatenate([src_l, src_r]), dst])).to(dev)
+    stream = torch.cuda.current_stream(dev)
+    width, stride = Hkv * D, pool.k_cache(1).data_ptr() - pool.k_cache(0).data_ptr() if layers > 1 else 0
+    from async_llm_amd import native
+
+    def launches():
+        for first, n, shift in ((0, n_left, 0), (n_left, n_right, left.mrope_span)):
+            native.check(native.lib.va_copy_shift_kv(
+                pool.k_cache(0).data_ptr(), pool.v_cache(0).data_ptr(), width, stride // 2, layers,
+                tables[0, first:].data_ptr(), tables[1, first:].data_ptr(), n, shift, att._shape,
+                att._rope_descriptor(), stream.cuda_stream))
+
+    times = []
+    for i in range(warmup + steps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        launches()
+        b.record(stream)
+        b.synchronize()
+        if i >= warmup:
+            times.append(a.elapsed_time(b))
+    kern_ms = sum(times) / len(times)
+    alg_bytes = 4 * layers * Hkv * D * 2 * (n_left + n_right)
+    line = {
+        "metric": "block_merge_hbm_gbps", "value": round(alg_bytes / ms_per_step / 1e6, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "block_merge", "left_tokens": n_left, "right_tokens": n_right, "layers": layers,
+                   "kv_heads": Hkv, "head_dim": D, "page_size": P, "alg_bytes": alg_bytes},
+        "roofline": {"bound": "hbm", "achieved": round(alg_bytes / kern_ms / 1e6, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(alg_bytes / kern_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "copy_shift_kernel x2 (left copy, right copy + key shift)",
+                     "kernel_ms_avg": round(kern_ms, 4)},
+    }
+    if cpu:
+        from oracle import view_attention_oracle as O
+
+        n = 4096  # tokens of each block in the sample, one layer
+        k_cpu = pool.k_cache(0)[: 4 * n // P].cpu().reshape(-1, Hkv, D)
+        v_cpu = pool.v_cache(0)[: 4 * n // P].cpu().reshape(-1, Hkv, D)
+        rope = O.RopeSpec(D, table.cpu())
+        reps = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            O.copy_shift_kv(k_cpu, v_cpu, range(0, n), range(2 * n, 3 * n), 0, rope)
+            O.copy_shift_kv(k_cpu, v_cpu, range(n, 2 * n), range(3 * n, 4 * n), n, rope)
+            reps.append(time.perf_counter() - t0)
+        t = sorted(reps)[1]
+        line["cpu_baseline"] = {"value": round(4 * Hkv * D * 2 * 2 * n / t / 1e9, 3), "unit": "GB/s",
+                                "cores": torch.get_num_threads(), "kind": "port",
+                                "sample": f"two {n}-token blocks, one layer, {t:.3f} s per pass, torch CPU oracle, "
+                                          "median of 3"}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -193,6 +294,8 @@ def main() -> int:
     torch.cuda.set_device(dev)
     if args.workload == "copy_calibration":
         return copy_calibration(dev, args.steps)
+    if args.workload == "block_merge":
+        return block_merge(dev, args.steps, args.warmup, args.layers, not args.no_cpu_baseline)
     wl = build_workload(args.workload, dev, args.layers, args.kernel)
     layers = args.layers
 
