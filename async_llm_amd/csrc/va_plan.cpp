@@ -551,9 +551,11 @@ static int write_plan(const Built& b, const VaSubRequests* subs, const VaShape* 
     c.plan_words = (int32_t)va_plan_fixed_words(cap);
     c.workspace_bytes = va_workspace_bytes_for(cap_partials, shape->num_q_heads, shape->head_dim);
   }
-  if (plan_capacity_words < c.plan_words)
+  if (plan_capacity_words < c.plan_words) {
+    if (counts) *counts = c;  // the caller learns the size it needs
     return va_fail(VA_ERR_CAPACITY, "plan needs %d words, buffer holds %lld", c.plan_words,
                    (long long)plan_capacity_words);
+  }
   int32_t* h = plan_host;
   std::memset(h, 0, sizeof(int32_t) * (size_t)c.plan_words);
   int32_t off = VA_PLAN_HEADER_WORDS;

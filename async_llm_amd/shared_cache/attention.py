@@ -33,7 +33,7 @@ import numpy as np
 import torch
 
 from .. import native
-from .attention_metadata import page_numbers, upload_page_indices
+from .attention_metadata import page_numbers_array, upload_page_indices
 from .rope_correction import rope_rows
 
 
@@ -180,6 +180,7 @@ class SharedCacheAttention:
         self._rope_desc: Optional[native.VaRope] = None
         self._workspace: Optional[torch.Tensor] = None
         self._workspace_prepared = False
+        self._plan_scratch = np.empty(1 << 16, dtype=np.int32)  # host scratch of the planner, grown on demand
 
     # ------------------------------------------------------------------
     # rotation
@@ -245,12 +246,19 @@ class SharedCacheAttention:
             arrays[0].ctypes.data, arrays[1].ctypes.data, arrays[2].ctypes.data if arrays[2].size else None,
             arrays[3].ctypes.data, arrays[4].ctypes.data, arrays[5].ctypes.data,
             sw.ctypes.data if sw.size else None)
+        # one pass of the planner: build into a scratch that is normally large enough, then copy
+        # the blob to pinned staging of its exact size
         counts = native.VaPlanCounts()
-        native.check(native.lib.va_plan_count(subs, self._shape, self.plan_params, counts))
+        scratch = self._plan_scratch
+        rc = native.lib.va_plan_build(subs, self._shape, self.plan_params, scratch.ctypes.data, scratch.size, counts)
+        if rc == native.VA_ERR_CAPACITY and counts.plan_words > scratch.size:
+            scratch = self._plan_scratch = np.empty(2 * counts.plan_words, dtype=np.int32)
+            rc = native.lib.va_plan_build(subs, self._shape, self.plan_params, scratch.ctypes.data, scratch.size,
+                                          counts)
+        native.check(rc)
         pin = self.device.type == "cuda"
         host = torch.empty(counts.plan_words, dtype=torch.int32, pin_memory=pin)
-        native.check(native.lib.va_plan_build(subs, self._shape, self.plan_params, host.data_ptr(),
-                                              counts.plan_words, counts))
+        host.numpy()[:] = scratch[: counts.plan_words]
         blob = host.to(self.device, non_blocking=True)
         refs.extend((host, blob))
         header = host[: native.PLAN_HEADER_WORDS].numpy().copy()
@@ -263,7 +271,7 @@ class SharedCacheAttention:
         assert W > 0
         P = self.page_size
         written = set(new_page_for_block)
-        snapshot: Dict[int, List[int]] = {}
+        snapshot: Dict[int, np.ndarray] = {}
         views, targets = group.cache_structure, group.write_to
 
         main = {"worker": [], "loc": [], "slot": [], "pages": [], "n_pages": [], "len": [], "last": []}
@@ -280,7 +288,7 @@ class SharedCacheAttention:
             for b, g in zip(view, grow):
                 length = b.num_tokens + g
                 if length:
-                    pages = page_numbers(b, snapshot, new_page_for_block.get(id(b)))
+                    pages = page_numbers_array(b, snapshot, new_page_for_block.get(id(b)))
                     main["worker"].append(w)
                     main["loc"].append(total_span - before - 1)
                     main["slot"].append(seg)
@@ -382,7 +390,7 @@ class SharedCacheAttention:
         per context block and one causal sub-request over its own block."""
         P = self.page_size
         max_segments = max(len(s.context) + 1 for s in specs)
-        snapshot: Dict[int, List[int]] = {}
+        snapshot: Dict[int, np.ndarray] = {}
 
         ctx = {"rows": [], "slot": [], "loc": [], "pages": [], "n_pages": [], "q": [], "len": [], "last": [],
                "chain": []}
@@ -405,7 +413,7 @@ class SharedCacheAttention:
                 ctx["rows"].append(rows)
                 ctx["slot"].append(np.full(S, j, dtype=np.int64))
                 ctx["loc"].append(rel + (first_new - ahead))
-                ctx["pages"].append(page_numbers(block, snapshot))
+                ctx["pages"].append(page_numbers_array(block, snapshot))
                 ctx["n_pages"].append(block.num_pages)
                 ctx["q"].append(S)
                 ctx["len"].append(block.num_tokens)

@@ -30,7 +30,7 @@ import numpy as np
 import torch
 
 from .. import native
-from .attention_metadata import page_numbers
+from .attention_metadata import page_numbers_array
 
 
 class _FixedPlanBuffers:
@@ -165,8 +165,8 @@ class SharedDecodeAttentionBuffers(_FixedPlanBuffers):
         self._wait_for_staging()
         self.refs = []
         kv = self._kv_host.numpy()
-        flat = [page for part in parts for page in part]
-        kv[:n_entries] = flat
+        if n_entries:
+            np.concatenate([np.asarray(part, dtype=np.int32) for part in parts if len(part)], out=kv[:n_entries])
         kv[n_entries:n_entries + w] = self.dummy_cpu
         loc = self._loc_host.numpy()
         valid = self._valid_host.numpy()
@@ -260,7 +260,7 @@ class SharedPrefillAttentionBuffers(_FixedPlanBuffers):
                 assert block.num_tokens > 0, "context blocks must be non-empty"
                 i = worker * d + slot
                 q_len[i], lengths[i], chain[i] = n, block.num_tokens, worker
-                pages[i] = page_numbers(block, snapshot)
+                pages[i] = page_numbers_array(block, snapshot)
                 gather.append(source)
                 slots.append(source * (d + 1) + slot)
                 locations.append(rel + position)
@@ -281,7 +281,9 @@ class SharedPrefillAttentionBuffers(_FixedPlanBuffers):
 
         self._wait_for_staging()
         self.refs = []
-        self._kv_host.numpy()[:n_entries] = [page for part in pages for page in part]
+        if n_entries:
+            np.concatenate([np.asarray(part, dtype=np.int32) for part in pages if len(part)],
+                           out=self._kv_host.numpy()[:n_entries])
         active = np.concatenate(slots) if slots else np.empty(0, dtype=np.int64)
         unused = np.ones(r * (d + 1), dtype=bool)
         unused[active] = False

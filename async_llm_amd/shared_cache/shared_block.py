@@ -90,7 +90,8 @@ class CacheBlock:
         self.block_id = next(_block_ids)
         self.device = device
         self.page_size = page_size
-        self.page_starts: List[int] = []
+        self._pages_version = 0  # bumped by every change of the page list: keys the planners' page-table cache
+        self.page_starts = []
         self.num_tokens: int = 0
         self.token_ids: List[int] = []
         self.mrope_span_override: Optional[int] = None
@@ -124,6 +125,16 @@ class CacheBlock:
     def _replace_linear_states(self, affine, conv) -> None:
         self.linear_affine = StateDict(self._gdn_state_cache, affine)
         self.linear_conv_state = StateDict(self._gdn_state_cache, conv)
+
+    # -- page list --------------------------------------------------------
+    @property
+    def page_starts(self) -> List[int]:
+        return self._page_starts
+
+    @page_starts.setter
+    def page_starts(self, value: List[int]) -> None:
+        self._page_starts = value
+        self._pages_version += 1
 
     # -- page arithmetic --------------------------------------------------
     @property
@@ -192,6 +203,7 @@ class CacheBlock:
         else:
             assert not self.has_capacity, "append_token got a new page but last page has room"
             self.page_starts.append(int(new_page_start))
+            self._pages_version += 1
         self.num_tokens += 1
         if self.mrope_span_override is not None:
             # decoded tokens are text: the frame advances by one with them
@@ -202,6 +214,7 @@ class CacheBlock:
         self.invalidate_gdn_state()
         released = list(self.page_starts)
         self.page_starts.clear()
+        self._pages_version += 1
         self.token_ids.clear()
         self.num_tokens = 0
         self.mrope_span_override = None

@@ -176,7 +176,9 @@ VA_API int va_plan_count(const VaSubRequests* subs, const VaShape* shape, const 
  * Items are in launch order, laid out for the 8 dies of an MI355X (workgroup b
  * of a launch runs on die b % 8): wide items first, then narrow ones, each
  * class padded with empty items (n_q = 0) to a multiple of 8; n_items and
- * n_wide_items count the padding.
+ * n_wide_items count the padding.  A caller may skip va_plan_count and build
+ * into a buffer of its own guess: when it is too small the call returns
+ * VA_ERR_CAPACITY and *counts holds the size to retry with.
  */
 VA_API int va_plan_build(const VaSubRequests* subs, const VaShape* shape, const VaPlanParams* params,
                   int32_t* plan_host, int64_t plan_capacity_words, VaPlanCounts* counts);

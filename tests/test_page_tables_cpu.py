@@ -283,3 +283,42 @@ def test_prepare_rejects_bad_input():
         a.prepare_prefill_batch([PrefillSpec([], torch.tensor([0]), 2, mrope_rel=torch.zeros(3, 5))])
     with pytest.raises(ValueError, match="kernel"):
         make_op(4, kernel="cuda")
+
+
+def test_page_array_cache_follows_every_change_of_the_page_list():
+    """The planners keep each block's page numbers as an array between prepares;
+    the array must equal the list-built table after every kind of change a
+    session makes to a block (reference shared_block.py grow/append/clear,
+    session.py:352 assignment), and foreign block objects are never cached."""
+    from async_llm_amd.shared_cache.attention_metadata import page_array, page_numbers_array
+
+    page = 4
+    b = CacheBlock(torch.device("cpu"), page)
+
+    def check():
+        want = page_numbers(b, {})
+        got = page_array(b)
+        assert got.dtype.name == "int32" and got.tolist() == want
+        assert page_numbers_array(b, {}, 40).tolist() == want + [10]
+        assert page_array(b) is got  # served from the cache while nothing changes
+
+    check()
+    b.grow_pages(torch.tensor([8, 20]), 7)
+    check()
+    b.append_token(None)
+    check()
+    b.append_token(32)  # opens a page
+    check()
+    b.page_starts = [4, 12, 16]  # a session assigning a fresh list (merge)
+    b.num_tokens = 12
+    check()
+    b.page_starts = [4, 12, 36]  # same length, different content
+    check()
+    b.clear()
+    check()
+    b.grow_pages(torch.tensor([4, 12, 36]), 9)
+    check()
+    foreign = SimpleNamespace(page_starts=[8, 4], page_size=page)
+    first = page_array(foreign)
+    foreign.page_starts[0] = 16  # changed in place, no version counter: must be seen
+    assert first.tolist() == [2, 1] and page_array(foreign).tolist() == [4, 1]
