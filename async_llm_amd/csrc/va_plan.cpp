@@ -74,7 +74,6 @@ int check_subs(const VaSubRequests* s, const VaShape* shape) {
       return va_fail(VA_ERR_ARG, "sub-request %d: seq_len %d does not fit its %d kv entries", i, len, ne);
     if ((s->flags[i] & VA_SUB_CAUSAL) && nq > len)
       return va_fail(VA_ERR_ARG, "sub-request %d: causal with more query rows (%d) than keys (%d)", i, nq, len);
-    if (ne > 0 && !s->kv_indices) return va_fail(VA_ERR_ARG, "null kv_indices");
   }
   for (int32_t i = 0; i < s->n_subrows; ++i)
     if (s->sub_worker[i] < 0 || s->sub_worker[i] >= s->n_rows)
@@ -157,7 +156,10 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
       const int32_t b = s->kv_indptr[i], ne = s->kv_indptr[i + 1] - b;
       int32_t gid = -1;
       uint64_t h = 0;
-      if (q_tile > 1) {
+      // readers are batched by comparing their KV lists; without a host copy of the lists
+      // (kv_indices == NULL) every sub-request stands alone
+      const bool can_group = q_tile > 1 && s->kv_indices && ne > 0;
+      if (can_group) {
         h = (uint64_t)(uint32_t)s->kv_indices[b] * 0x9E3779B97F4A7C15ull ^
             ((uint64_t)(uint32_t)s->seq_lens[i] << 32) ^ (uint64_t)(uint32_t)(ne * 31 + s->flags[i]);
         auto it = by_hash.find(h);
@@ -176,7 +178,7 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
       if (gid < 0) {
         gid = (int32_t)groups.size();
         groups.push_back(Group{i, {}});
-        if (q_tile > 1) by_hash[h].push_back(gid);
+        if (can_group) by_hash[h].push_back(gid);
       }
       for (int32_t r = s->qo_indptr[i]; r < s->qo_indptr[i + 1]; ++r) groups[gid].subrows.push_back(r);
     }

@@ -186,6 +186,9 @@ class SharedCacheAttention:
     # rotation
     # ------------------------------------------------------------------
     def _rope_descriptor(self) -> native.VaRope:
+        if self._rope_desc is None and self.rotary_dim == 0:
+            # nothing rotates (queries and keys arrive rotated): no table is needed
+            self._rope_desc = native.VaRope(native.VA_ROPE_TABLE, 0, None, 0, 0, 0, None)
         if self._rope_desc is None:
             table = None
             if self.mrope_section is None:

@@ -133,7 +133,8 @@ typedef struct VaSubRequests {
   int32_t n_rows;             /* output rows (workers / new tokens) */
   const int32_t* qo_indptr;   /* [n_sub+1] host */
   const int32_t* kv_indptr;   /* [n_sub+1] host */
-  const int32_t* kv_indices;  /* [kv_indptr[n_sub]] host */
+  const int32_t* kv_indices;  /* [kv_indptr[n_sub]] host; NULL when the table only exists on the
+                                 device: readers of one KV list are then not batched into shared tiles */
   const int32_t* seq_lens;    /* [n_sub] host */
   const int32_t* flags;       /* [n_sub] host */
   const int32_t* chain;       /* [n_sub] host */
