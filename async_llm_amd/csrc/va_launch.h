@@ -16,6 +16,7 @@ struct AttnArgs {
   const int32_t* items;
   const int32_t* links;
   const int32_t* qrefs;
+  const int32_t* qref_rows;  // sub_worker[qrefs[k]], precomputed by the planner
   const int32_t* kv_indices;
   const int64_t* sub_worker;
   const int64_t* sub_loc;

@@ -66,6 +66,17 @@ __device__ __forceinline__ int swz(int r) {
   return (r >> 1) & 7;
 }
 
+#if VA_STREAM_TIMELINE  // experiment builds: per-workgroup start, set-up end, loop end, end, hardware id
+__device__ unsigned long long va_debug_times[8 * 16384];
+extern "C" __attribute__((visibility("default"))) int va_debug_read(void* host, size_t bytes) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(va_debug_times), bytes);
+}
+#define VA_STAMP(k) \
+  if (threadIdx.x == 0 && blockIdx.x < 16384) va_debug_times[8 * blockIdx.x + (k)] = wall_clock64();
+#else
+#define VA_STAMP(k)
+#endif
+
 template <typename E, int kD>
 __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void attn_stream_kernel(AttnArgs a) {
   using S = typename E::storage;
@@ -81,6 +92,12 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
   const int G = a.num_q_heads / a.num_kv_heads;
   const int n_q = item[VA_I_N_Q];
   if (n_q == 0) return;  // padding item: keeps the launch order aligned with the die round-robin
+  VA_STAMP(0)
+#if VA_STREAM_TIMELINE
+  if (threadIdx.x == 0 && blockIdx.x < 16384)
+    va_debug_times[8 * blockIdx.x + 4] = __builtin_amdgcn_s_getreg(4 | (31 << 11)) |
+                                         ((unsigned long long)__builtin_amdgcn_s_getreg(20 | (31 << 11)) << 32);
+#endif
   const int part_base = item[VA_I_PART_BASE];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -126,7 +143,8 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
   for (int t = 0; t < kRun; ++t) o[t] = va_f32x4{0.f, 0.f, 0.f, 0.f};
 
   for (int li = 0; li < item[VA_I_N_LINKS]; ++li) {
-    const int32_t* link = a.links + (long long)(item[VA_I_LINK_BEGIN] + li) * VA_LINK_WORDS;
+    // the first link travels with the item
+    const int32_t* link = li == 0 ? item + VA_I_LINK0 : a.links + (long long)(item[VA_I_LINK_BEGIN] + li) * VA_LINK_WORDS;
     const int lflags = link[VA_L_FLAGS];
     const int qref = link[VA_L_QREF];
     const int kv_begin = link[VA_L_KV_BEGIN];
@@ -150,8 +168,11 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     auto page_of = [&](int i) __attribute__((always_inline)) {
       return ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + ((tok_begin + i * kStreamTok) >> p_shift)];
     };
-    auto issue = [&](int i, auto uniform_tag, int page) __attribute__((always_inline)) {
+    // `both_tag`: the wave (0 or 1, which own the K loads) also issues the V loads of waves 2 and 3,
+    // whose lane pattern is the same; used for the first tiles of a link.
+    auto issue = [&](int i, auto uniform_tag, int page, auto both_tag) __attribute__((always_inline)) {
       constexpr bool kUniform = decltype(uniform_tag)::value;
+      constexpr bool kBoth = decltype(both_tag)::value;
       const int t0 = tok_begin + i * kStreamTok;
       va_u32x4* buf = ring + (i % kBuffers) * 2 * kTileUnits;
       long long base_byte = 0;  // wave-uniform: pool byte offset of the tile's first token
@@ -162,44 +183,55 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
 #pragma unroll
       for (int u = 0; u < Sh::kLoadsPerWave; ++u) {
         const int q = wave * Sh::kLoadsPerWave + u;  // wave-uniform
-        const bool is_v = q >= Sh::kLoadsPerKind;
-        const int first_row = (is_v ? q - Sh::kLoadsPerKind : q) * Sh::kRowsPerLoad;
         const int r = min(ld_row[u], last_row);
-        const char* src;
+        long long row_byte;
         if constexpr (kUniform) {
-          src = (const char*)(is_v ? vp : kp) + base_byte + (uint32_t)(r * row_bytes + ld_byte[u]);
+          row_byte = base_byte + (uint32_t)(r * row_bytes + ld_byte[u]);
         } else {
-          src = (const char*)(is_v ? vp : kp) + kv_slot(a.kv_indices, kv_begin, t0 + r, P, slots) * row_bytes +
-                ld_byte[u];
+          row_byte = kv_slot(a.kv_indices, kv_begin, t0 + r, P, slots) * row_bytes + ld_byte[u];
         }
-        const va_u32x4* dst = buf + (is_v ? kTileUnits : 0) + first_row * kChunks;  // + lane, implied by the load
-        load_to_lds(src, __builtin_amdgcn_readfirstlane(lds_address(dst)));
+#pragma unroll
+        for (int kind = 0; kind < (kBoth ? 2 : 1); ++kind) {
+          const bool is_v = kBoth ? kind == 1 : q >= Sh::kLoadsPerKind;
+          const int first_row = ((!kBoth && is_v) ? q - Sh::kLoadsPerKind : q) * Sh::kRowsPerLoad;
+          const va_u32x4* dst = buf + (is_v ? kTileUnits : 0) + first_row * kChunks;  // + lane, implied by the load
+          load_to_lds((const char*)(is_v ? vp : kp) + row_byte, __builtin_amdgcn_readfirstlane(lds_address(dst)));
+        }
       }
     };
 
     // ---- set-up: first tiles on their way, then the query tile ----
+    // The two halves of the workgroup split the work: waves 0 and 1 request the first tiles (K and
+    // V), waves 2 and 3 rotate the query tile.  Loads complete in order per wave, so a wave that
+    // did both would find its query rows only after its share of the tiles had arrived, at every
+    // step of the chain of dependent loads that leads to them.
     __syncthreads();  // every wave is done with the previous link's buffers
     auto first_tiles = [&](auto uniform_tag) __attribute__((always_inline)) {
 #pragma unroll
       for (int i = 0; i < kBuffers - 1; ++i)
-        if (i < n_tiles) issue(i, uniform_tag, decltype(uniform_tag)::value ? page_of(i) : 0);
+        if (i < n_tiles) issue(i, uniform_tag, decltype(uniform_tag)::value ? page_of(i) : 0, std::true_type{});
     };
-    if (uniform_pages) {
-      first_tiles(std::true_type{});
-    } else {
-      first_tiles(std::false_type{});
+    if (wave < 2) {
+      if (uniform_pages) {
+        first_tiles(std::true_type{});
+      } else {
+        first_tiles(std::false_type{});
+      }
     }
 
+    VA_STAMP(5)
     // rotate the query tile into the last buffer (not yet in use), swizzled like a K tile
     va_u32x4* q_stage = ring + (kBuffers - 1) * 2 * kTileUnits;
-    for (int idx = tid; idx < 16 * (kChunks / 2); idx += kStreamThreads) {  // two pieces per step
+    for (int idx = tid - 2 * kWave; idx >= 0 && idx < 16 * (kChunks / 2); idx += 2 * kWave) {  // two pieces per step
       const int jr = idx / (kChunks / 2), x = idx - jr * (kChunks / 2);
       const int iq = jr / G, g = jr - iq * G;
       int c0 = 2 * x, c1 = 2 * x + 1;
       uint4 p0 = make_uint4(0, 0, 0, 0), p1 = p0;
       if (iq < n_q) {
-        const int subrow = (lflags & VA_LINK_INDIRECT) ? a.qrefs[qref + iq] : qref + iq;
-        const long long src_row = a.sub_worker[subrow];
+        // indirect links find sub-row and query row side by side in the plan; direct ones ask sub_worker
+        const bool indirect = lflags & VA_LINK_INDIRECT;
+        const int subrow = indirect ? a.qrefs[qref + iq] : qref + iq;
+        const long long src_row = indirect ? (long long)a.qref_rows[qref + iq] : a.sub_worker[subrow];
         const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
         const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
         rotated_query_unit<E>(a.rope, qh, x, p, c0, c1, p0, p1);
@@ -207,15 +239,18 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
       q_stage[jr * kChunks + (c0 ^ swz<kD>(jr))] = va_u32x4{p0.x, p0.y, p0.z, p0.w};
       q_stage[jr * kChunks + (c1 ^ swz<kD>(jr))] = va_u32x4{p1.x, p1.y, p1.z, p1.w};
     }
+    VA_STAMP(6)
     ring_barrier<kAnyInFlight>();
+    VA_STAMP(7)
     va_u32x4 qf[kSteps];  // B operands: row j, dims [32s + 8kg, +8)
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) qf[s] = q_stage[j * kChunks + ((4 * s + kg) ^ swz<kD>(j))];
     ring_barrier<kAnyInFlight>();  // the staging buffer may be refilled now
+    VA_STAMP(1)
 
     // ---- the tile loop, once per page-table kind so neither carries the other's branches ----
     auto stream = [&](auto uniform_tag) __attribute__((always_inline)) {
-    if (kBuffers - 1 < n_tiles) issue(kBuffers - 1, uniform_tag, decltype(uniform_tag)::value ? page_of(kBuffers - 1) : 0);
+    if (kBuffers - 1 < n_tiles) issue(kBuffers - 1, uniform_tag, decltype(uniform_tag)::value ? page_of(kBuffers - 1) : 0, std::false_type{});
     for (int i = 0; i < n_tiles; ++i) {
       // This wave's loads of tile i have landed once at most the loads of the tiles requested
       // after it are outstanding; the barrier then covers the other waves' loads.
@@ -288,7 +323,7 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
       // refill this tile's buffer once every wave has consumed it
       if (refill) {
         ring_barrier<kAnyInFlight>();
-        issue(i + kBuffers, uniform_tag, next_page);
+        issue(i + kBuffers, uniform_tag, next_page, std::false_type{});
       }
     }
     };
@@ -299,6 +334,7 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     }
   }
 
+  VA_STAMP(2)
   // row sums live spread over the four contraction groups
   l_run += __shfl_xor(l_run, 16, kWave);
   l_run += __shfl_xor(l_run, 32, kWave);
@@ -309,10 +345,10 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     const int hq = hk * G + g;
     const int d0 = wave * Sh::kDimsPerWave + 4 * kRun * kg;
     if (part_base < 0) {
-      const int32_t* link0 = a.links + (long long)item[VA_I_LINK_BEGIN] * VA_LINK_WORDS;
-      const int subrow =
-          (link0[VA_L_FLAGS] & VA_LINK_INDIRECT) ? a.qrefs[link0[VA_L_QREF] + row_iq] : link0[VA_L_QREF] + row_iq;
-      const long long out_row = a.sub_worker[subrow];
+      const int32_t* link0 = item + VA_I_LINK0;
+      const long long out_row = (link0[VA_L_FLAGS] & VA_LINK_INDIRECT)
+                                    ? (long long)a.qref_rows[link0[VA_L_QREF] + row_iq]
+                                    : a.sub_worker[link0[VA_L_QREF] + row_iq];
       S* orow = (S*)a.out + (out_row * a.num_q_heads + hq) * (long long)kD + d0;
       const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
       uint32_t w[2 * kRun];
@@ -343,6 +379,7 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
       }
     }
   }
+  VA_STAMP(3)
 }
 
 template <typename E, int kD>

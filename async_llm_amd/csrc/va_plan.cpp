@@ -292,10 +292,17 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     };
     // narrow tiles: chunk-major; wide tiles: their own (finer) chunking
     const int32_t per = chunk_len(kv_chunk);
-    for (int32_t t0 = 0; t0 < len; t0 += per) {
+    // The last chunk of a run is cut in two: every run then contributes short items, which the
+    // launch order puts last, so the launch does not end on a round of full-length items.
+    std::vector<int32_t> cuts{0};
+    for (int32_t t0 = per; t0 < len; t0 += per) cuts.push_back(t0);
+    if (len - cuts.back() >= 4 * gran) cuts.push_back(cuts.back() + round_up((len - cuts.back()) / 2, gran));
+    cuts.push_back(len);
+    for (size_t ci = 0; ci + 1 < cuts.size(); ++ci) {
+      if (cuts[ci] >= cuts[ci + 1]) continue;
       const int32_t unit = next_unit++;  // the narrow tiles of one chunk: same die, side by side
       for (size_t ti = 0; ti < tiles.size(); ++ti)
-        if (tiles[ti].second - tiles[ti].first <= q_tile) emit_range(ti, t0, std::min(len, t0 + per), unit);
+        if (tiles[ti].second - tiles[ti].first <= q_tile) emit_range(ti, cuts[ci], cuts[ci + 1], unit);
     }
     const int32_t per_w = chunk_len(wide_chunk);
     for (size_t ti = 0; ti < tiles.size(); ++ti)
@@ -504,7 +511,7 @@ void fill_counts(const Built& b, const VaSubRequests* s, const VaShape* shape, V
   c->n_partials = b.n_partials;
   c->n_row_parts = (int32_t)b.row_ids.size();
   c->plan_words = VA_PLAN_HEADER_WORDS + c->n_items * VA_ITEM_WORDS + c->n_links * VA_LINK_WORDS +
-                  c->n_qrefs + (s->n_rows + 1) + c->n_row_parts + s->n_rows;
+                  2 * c->n_qrefs + (s->n_rows + 1) + c->n_row_parts + s->n_rows;
   c->workspace_bytes = va_workspace_bytes_for(b.n_partials, shape->num_q_heads, shape->head_dim);
 }
 
@@ -585,6 +592,16 @@ static int write_plan(const Built& b, const VaSubRequests* subs, const VaShape* 
     w[VA_I_PART_BASE] = it.part_base;
     w[VA_I_TOKENS] = it.tokens;
     w[VA_I_KIND] = it.kind;
+    if (it.n_links > 0) {
+      const Link& l = b.links[it.link_begin];
+      int32_t* lw = w + VA_I_LINK0;
+      lw[VA_L_KV_BEGIN] = l.kv_begin;
+      lw[VA_L_TOK_BEGIN] = l.tok_begin;
+      lw[VA_L_TOK_END] = l.tok_end;
+      lw[VA_L_QREF] = l.qref;
+      lw[VA_L_CAUSAL_BASE] = l.causal_base;
+      lw[VA_L_FLAGS] = l.flags;
+    }
   };
   for (int32_t i = 0; i < b.n_wide; ++i) write_item(i, b.items[i]);
   for (int32_t i = b.n_wide; i < cap_wide; ++i) write_item(i, Item{0, 0, 0, -1, 0, 1, -1});
@@ -605,6 +622,9 @@ static int write_plan(const Built& b, const VaSubRequests* subs, const VaShape* 
   off += cap_links * VA_LINK_WORDS;
   h[VA_H_OFF_QREFS] = off;
   std::copy(b.qrefs.begin(), b.qrefs.end(), plan_host + off);
+  off += cap_qrefs;
+  h[VA_H_OFF_QREF_ROWS] = off;
+  for (size_t i = 0; i < b.qrefs.size(); ++i) plan_host[off + i] = (int32_t)subs->sub_worker[b.qrefs[i]];
   off += cap_qrefs;
   h[VA_H_OFF_ROW_INDPTR] = off;
   std::copy(b.row_indptr.begin(), b.row_indptr.end(), plan_host + off);
@@ -633,14 +653,15 @@ extern "C" int va_plan_build(const VaSubRequests* subs, const VaShape* shape, co
 extern "C" int64_t va_plan_fixed_words(const VaPlanCapacity* cap) {
   if (!cap) return 0;
   return (int64_t)VA_PLAN_HEADER_WORDS + ((int64_t)cap->max_items + cap->max_wide_items) * VA_ITEM_WORDS +
-         (int64_t)cap->max_links * VA_LINK_WORDS + cap->max_qrefs + (cap->max_rows + 1) + cap->max_row_parts +
-         cap->max_rows;
+         (int64_t)cap->max_links * VA_LINK_WORDS + 2 * (int64_t)cap->max_qrefs + (cap->max_rows + 1) +
+         cap->max_row_parts + cap->max_rows;
 }
 
 // Upper bounds of every plan section for a workload within `lim`, following the rules of build():
 //   * stand-alone sub-requests: a group of readers is cut into tiles x chunks with
-//     chunk >= total_tokens / target, so items <= tiles + target with tiles <= sub-requests; every
-//     item carries one link; a query row enters the partial list once per chunk of its run;
+//     chunk >= total_tokens / target, plus one for the halved last chunk, so items <= 2 tiles + target
+//     with tiles <= sub-requests; every item carries one link; a query row enters the partial list
+//     once per chunk of its run;
 //   * chains: tiles of up to wide_tile rows (the last one of a chain may be narrow), each split
 //     into at most ceil(target / tiles) pieces, so items <= tiles + target per class; a tile has
 //     one link per member plus one per cut; a split tile's rows enter the partial list once per piece.
@@ -672,13 +693,13 @@ extern "C" int va_plan_capacity(const VaShape* shape, const VaPlanParams* params
 
   int64_t narrow = 0, wide = 0, links = 0, qrefs = 0, partials = 0;
   if (subs > 0) {
-    narrow += sub_rows + target;  // tiles <= query rows
+    narrow += 2 * sub_rows + target;  // tiles <= query rows; the halved last chunk adds one item per tile
     // wide decode tiles are cut at min(chunk, their tokens / (256 / kv heads))
     if (wide_groups) wide += sub_rows + target + 256;
     qrefs += sub_rows;
     // a query row is in one tile; that tile has at most 1 + len / chunk chunks, and the sum of
     // len / chunk over tiles is at most target (times the tile's rows when counted per row)
-    partials += sub_rows + (q_tile + (wide_groups ? wide_tile : 0)) * (target + 256);
+    partials += 2 * sub_rows + (q_tile + (wide_groups ? wide_tile : 0)) * (target + 256);
   }
   if (chains > 0 && chain_rows > 0) {
     const int64_t tile_rows = wide_tile ? wide_tile : q_tile;

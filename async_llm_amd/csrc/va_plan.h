@@ -10,7 +10,7 @@
 
 #define VA_PLAN_MAGIC 0x56415031  // "VAP1"
 #define VA_PLAN_HEADER_WORDS 24
-#define VA_ITEM_WORDS 8
+#define VA_ITEM_WORDS 16
 #define VA_LINK_WORDS 8
 
 // header word indices
@@ -35,6 +35,7 @@ enum {
   VA_H_N_SUBROWS,
   VA_H_N_WIDE,     // items [0, n_wide) are wide tiles, the rest narrow
   VA_H_WIDE_TILE,
+  VA_H_OFF_QREF_ROWS,  // parallel to qrefs: the query/output row of each entry (sub_worker[qrefs[k]])
 };
 
 // item word indices
@@ -45,6 +46,8 @@ enum {
   VA_I_PART_BASE,  // first partial slot (one per query row), or -1: write `out` directly
   VA_I_TOKENS,     // KV tokens the item walks (scheduling weight)
   VA_I_KIND,       // 1: wide tile (more rows than the streaming kernel's tile)
+  VA_I_LINK0 = 8,  // words 8..15: a copy of the item's first link, so that a kernel finds it with the
+                   // same load as the item (one level less in the chain of dependent loads at its start)
 };
 
 // link word indices

@@ -497,6 +497,7 @@ extern "C" int va_attention(const void* q_dev, int64_t q_row_stride, const void*
   a.items = plan_dev + h[VA_H_OFF_ITEMS];
   a.links = plan_dev + h[VA_H_OFF_LINKS];
   a.qrefs = plan_dev + h[VA_H_OFF_QREFS];
+  a.qref_rows = plan_dev + h[VA_H_OFF_QREF_ROWS];
   a.kv_indices = kv_indices_dev;
   a.sub_worker = sub_worker_dev;
   a.sub_loc = sub_loc_dev;

@@ -172,8 +172,11 @@ VA_API int va_plan_count(const VaSubRequests* subs, const VaShape* shape, const 
  * Build the plan into plan_host (capacity plan_capacity_words int32 words, at
  * least counts->plan_words).  The blob is position independent: copy it to the
  * device verbatim and pass the device copy to va_attention.  Layout (int32
- * words): header[24] | items[n_items*8] | links[n_links*8] | qrefs[n_qrefs] |
- * row_part_indptr[n_rows+1] | row_part_ids[n_row_parts] | row_flags[n_rows].
+ * words): header[24] | items[n_items*16] | links[n_links*8] | qrefs[n_qrefs] |
+ * qref_rows[n_qrefs] | row_part_indptr[n_rows+1] | row_part_ids[n_row_parts] |
+ * row_flags[n_rows].  (An item carries a copy of its first link, and qref_rows
+ * the output row of every qrefs entry: both shorten the chain of dependent loads
+ * at the start of a workgroup.)
  * Items are in launch order, laid out for the 8 dies of an MI355X (workgroup b
  * of a launch runs on die b % 8): wide items first, then narrow ones, each
  * class padded with empty items (n_q = 0) to a multiple of 8; n_items and

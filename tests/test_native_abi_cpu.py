@@ -15,7 +15,7 @@ from async_llm_amd import native
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 H = dict(MAGIC=0, KERNEL=1, Q_TILE=2, KV_CHUNK=3, N_ITEMS=4, N_LINKS=5, N_QREFS=6, N_PARTIALS=7, N_ROW_PARTS=8,
          N_ROWS=9, OFF_ITEMS=10, OFF_LINKS=11, OFF_QREFS=12, OFF_ROW_INDPTR=13, OFF_ROW_IDS=14, OFF_ROW_FLAGS=15,
-         N_EMPTY=16, N_SUBROWS=17, N_WIDE=18, WIDE_TILE=19)
+         N_EMPTY=16, N_SUBROWS=17, N_WIDE=18, WIDE_TILE=19, OFF_QREF_ROWS=20)
 NO_CAUSAL = 0x3FFFFFFF
 
 
@@ -52,7 +52,7 @@ def build_plan(qo, kvp, kvi, lens, flags, chain, sub_worker, n_rows, heads=(8, 2
 def decode_plan(blob):
     h = blob[: native.PLAN_HEADER_WORDS]
     assert h[H["MAGIC"]] == 0x56415031
-    items = blob[h[H["OFF_ITEMS"]]: h[H["OFF_ITEMS"]] + 8 * h[H["N_ITEMS"]]].reshape(-1, 8)
+    items = blob[h[H["OFF_ITEMS"]]: h[H["OFF_ITEMS"]] + 16 * h[H["N_ITEMS"]]].reshape(-1, 16)
     links = blob[h[H["OFF_LINKS"]]: h[H["OFF_LINKS"]] + 8 * h[H["N_LINKS"]]].reshape(-1, 8)
     qrefs = blob[h[H["OFF_QREFS"]]: h[H["OFF_QREFS"]] + h[H["N_QREFS"]]]
     n_rows = h[H["N_ROWS"]]
@@ -85,6 +85,7 @@ def check_coverage(blob, qo, kvp, lens, flags, sub_worker, n_rows, fixed=False):
             continue
         assert nl >= 1 and 1 <= nq <= max(h[H["Q_TILE"]], h[H["WIDE_TILE"]])
         assert it[5] == int(nq > h[H["Q_TILE"]])  # kind: wide iff more rows than the narrow tile
+        assert list(it[8:14]) == list(links[lb][:6])  # the item carries a copy of its first link
         rows_of_item = None
         for l in links[lb: lb + nl]:
             kv_begin, t0, t1, qref, cbase, lflags = l[:6]
@@ -92,6 +93,8 @@ def check_coverage(blob, qo, kvp, lens, flags, sub_worker, n_rows, fixed=False):
             rows = []
             for i in range(nq):
                 sr = int(qrefs[qref + i]) if lflags & 1 else int(qref + i)
+                if lflags & 1:  # the row of an indirect entry is stored beside it
+                    assert blob[h[H["OFF_QREF_ROWS"]] + qref + i] == sub_worker[sr]
                 s = sub_of_row[sr]
                 assert kvp[s] == kv_begin or lens[s] == lens[[x for x in range(len(lens)) if kvp[x] == kv_begin][0]]
                 assert t1 <= lens[s]
@@ -225,7 +228,8 @@ def test_readers_of_one_block_share_a_tile():
     rc, blob, counts = build_plan(qo, kvp, kvi, lens, flags, chain, sw, 6, page=page, q_tile=4, kv_chunk=1024)
     assert rc == 0
     h, items, links, qrefs, *_ = decode_plan(blob)
-    assert sorted(int(i[2]) for i in items if i[2]) == [2, 4]  # 6 readers -> tiles of 4 and 2 rows, one chunk each
+    # 6 readers -> tiles of 4 and 2 rows; the run is one chunk, cut in two (192 + 108 tokens)
+    assert sorted((int(i[2]), int(i[4])) for i in items if i[2]) == [(2, 108), (2, 192), (4, 108), (4, 192)]
     check_coverage(blob, qo, kvp, lens, flags, sw, 6)
 
 
@@ -258,7 +262,8 @@ def test_tiles_of_one_chunk_run_on_one_die():
         load[pos % 8] += int(it[4])
         if l[0] == 0:  # kv_begin of the shared block's representative
             where.setdefault(int(l[1]), []).append(pos)
-    assert len(where) == L // 256 and all(len(v) == n_req // 4 for v in where.values())
+    # 8 chunks of 256 tokens, the last one cut in two
+    assert len(where) == L // 256 + 1 and all(len(v) == n_req // 4 for v in where.values())
     for t0, positions in where.items():
         assert len({p % 8 for p in positions}) == 1, (t0, positions)
         slots = sorted(p // 8 for p in positions)
