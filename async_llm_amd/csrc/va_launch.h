@@ -16,7 +16,6 @@ struct AttnArgs {
   const int32_t* items;
   const int32_t* links;
   const int32_t* qrefs;
-  const int32_t* qref_rows;  // sub_worker[qrefs[k]], precomputed by the planner
   const int32_t* kv_indices;
   const int64_t* sub_worker;
   const int64_t* sub_loc;
@@ -29,6 +28,7 @@ struct AttnArgs {
   int num_q_heads, num_kv_heads, head_dim, page_size;
   RopeDev rope;
   float scale_log2;  // log2(e) / sqrt(head_dim)
+  const int32_t* qref_rows;  // sub_worker[qrefs[k]], precomputed by the planner
 };
 
 struct MergeArgs {

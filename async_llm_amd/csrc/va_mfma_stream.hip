@@ -168,11 +168,8 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     auto page_of = [&](int i) __attribute__((always_inline)) {
       return ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + ((tok_begin + i * kStreamTok) >> p_shift)];
     };
-    // `both_tag`: the wave (0 or 1, which own the K loads) also issues the V loads of waves 2 and 3,
-    // whose lane pattern is the same; used for the first tiles of a link.
-    auto issue = [&](int i, auto uniform_tag, int page, auto both_tag) __attribute__((always_inline)) {
+    auto issue = [&](int i, auto uniform_tag, int page) __attribute__((always_inline)) {
       constexpr bool kUniform = decltype(uniform_tag)::value;
-      constexpr bool kBoth = decltype(both_tag)::value;
       const int t0 = tok_begin + i * kStreamTok;
       va_u32x4* buf = ring + (i % kBuffers) * 2 * kTileUnits;
       long long base_byte = 0;  // wave-uniform: pool byte offset of the tile's first token
@@ -183,46 +180,37 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
 #pragma unroll
       for (int u = 0; u < Sh::kLoadsPerWave; ++u) {
         const int q = wave * Sh::kLoadsPerWave + u;  // wave-uniform
+        const bool is_v = q >= Sh::kLoadsPerKind;
+        const int first_row = (is_v ? q - Sh::kLoadsPerKind : q) * Sh::kRowsPerLoad;
         const int r = min(ld_row[u], last_row);
-        long long row_byte;
+        const char* src;
         if constexpr (kUniform) {
-          row_byte = base_byte + (uint32_t)(r * row_bytes + ld_byte[u]);
+          src = (const char*)(is_v ? vp : kp) + base_byte + (uint32_t)(r * row_bytes + ld_byte[u]);
         } else {
-          row_byte = kv_slot(a.kv_indices, kv_begin, t0 + r, P, slots) * row_bytes + ld_byte[u];
+          src = (const char*)(is_v ? vp : kp) + kv_slot(a.kv_indices, kv_begin, t0 + r, P, slots) * row_bytes +
+                ld_byte[u];
         }
-#pragma unroll
-        for (int kind = 0; kind < (kBoth ? 2 : 1); ++kind) {
-          const bool is_v = kBoth ? kind == 1 : q >= Sh::kLoadsPerKind;
-          const int first_row = ((!kBoth && is_v) ? q - Sh::kLoadsPerKind : q) * Sh::kRowsPerLoad;
-          const va_u32x4* dst = buf + (is_v ? kTileUnits : 0) + first_row * kChunks;  // + lane, implied by the load
-          load_to_lds((const char*)(is_v ? vp : kp) + row_byte, __builtin_amdgcn_readfirstlane(lds_address(dst)));
-        }
+        const va_u32x4* dst = buf + (is_v ? kTileUnits : 0) + first_row * kChunks;  // + lane, implied by the load
+        load_to_lds(src, __builtin_amdgcn_readfirstlane(lds_address(dst)));
       }
     };
 
     // ---- set-up: first tiles on their way, then the query tile ----
-    // The two halves of the workgroup split the work: waves 0 and 1 request the first tiles (K and
-    // V), waves 2 and 3 rotate the query tile.  Loads complete in order per wave, so a wave that
-    // did both would find its query rows only after its share of the tiles had arrived, at every
-    // step of the chain of dependent loads that leads to them.
     __syncthreads();  // every wave is done with the previous link's buffers
     auto first_tiles = [&](auto uniform_tag) __attribute__((always_inline)) {
 #pragma unroll
       for (int i = 0; i < kBuffers - 1; ++i)
-        if (i < n_tiles) issue(i, uniform_tag, decltype(uniform_tag)::value ? page_of(i) : 0, std::true_type{});
+        if (i < n_tiles) issue(i, uniform_tag, decltype(uniform_tag)::value ? page_of(i) : 0);
     };
-    if (wave < 2) {
-      if (uniform_pages) {
-        first_tiles(std::true_type{});
-      } else {
-        first_tiles(std::false_type{});
-      }
+    if (uniform_pages) {
+      first_tiles(std::true_type{});
+    } else {
+      first_tiles(std::false_type{});
     }
 
-    VA_STAMP(5)
     // rotate the query tile into the last buffer (not yet in use), swizzled like a K tile
     va_u32x4* q_stage = ring + (kBuffers - 1) * 2 * kTileUnits;
-    for (int idx = tid - 2 * kWave; idx >= 0 && idx < 16 * (kChunks / 2); idx += 2 * kWave) {  // two pieces per step
+    for (int idx = tid; idx < 16 * (kChunks / 2); idx += kStreamThreads) {  // two pieces per step
       const int jr = idx / (kChunks / 2), x = idx - jr * (kChunks / 2);
       const int iq = jr / G, g = jr - iq * G;
       int c0 = 2 * x, c1 = 2 * x + 1;
@@ -239,9 +227,7 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
       q_stage[jr * kChunks + (c0 ^ swz<kD>(jr))] = va_u32x4{p0.x, p0.y, p0.z, p0.w};
       q_stage[jr * kChunks + (c1 ^ swz<kD>(jr))] = va_u32x4{p1.x, p1.y, p1.z, p1.w};
     }
-    VA_STAMP(6)
     ring_barrier<kAnyInFlight>();
-    VA_STAMP(7)
     va_u32x4 qf[kSteps];  // B operands: row j, dims [32s + 8kg, +8)
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) qf[s] = q_stage[j * kChunks + ((4 * s + kg) ^ swz<kD>(j))];
@@ -250,7 +236,7 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
 
     // ---- the tile loop, once per page-table kind so neither carries the other's branches ----
     auto stream = [&](auto uniform_tag) __attribute__((always_inline)) {
-    if (kBuffers - 1 < n_tiles) issue(kBuffers - 1, uniform_tag, decltype(uniform_tag)::value ? page_of(kBuffers - 1) : 0, std::false_type{});
+    if (kBuffers - 1 < n_tiles) issue(kBuffers - 1, uniform_tag, decltype(uniform_tag)::value ? page_of(kBuffers - 1) : 0);
     for (int i = 0; i < n_tiles; ++i) {
       // This wave's loads of tile i have landed once at most the loads of the tiles requested
       // after it are outstanding; the barrier then covers the other waves' loads.
@@ -323,7 +309,7 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
       // refill this tile's buffer once every wave has consumed it
       if (refill) {
         ring_barrier<kAnyInFlight>();
-        issue(i + kBuffers, uniform_tag, next_page, std::false_type{});
+        issue(i + kBuffers, uniform_tag, next_page);
       }
     }
     };
