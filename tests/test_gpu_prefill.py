@@ -152,3 +152,22 @@ def test_split_chains_with_unaligned_pieces(dtype):
         real = [it for it in items if it[2] > 0]
         assert len(real) > 1, "the chain was not split"
         assert any(l[1] % 16 for it in real for l in links[it[0]: it[0] + it[1]]), "no unaligned piece in this plan"
+
+
+@pytest.mark.parametrize("dtype,heads,rotary", [
+    (torch.bfloat16, (4, 4, 64), 64),      # one q head per kv head: 256-row wide tiles
+    (torch.bfloat16, (16, 2, 128), 64),    # 8 q heads per kv head, partial rotation
+    (torch.float16, (16, 1, 256), 256),    # 16 q heads per kv head: a wide tile is 8 requests rows
+    (torch.float16, (8, 4, 256), 128),     # 2 q heads per kv head at head_dim 256
+])
+def test_prefill_head_layouts(dtype, heads, rotary):
+    """Every supported ratio of q to kv heads through the wide and the streaming
+    kernel: tiles of 256/G (128/G at head_dim 256) rows, tails of at most 16/G."""
+    page = 16
+    op, cpu_pool, dev_pool, gen = make_op_and_pool(DEV, dtype, heads, page, 96, 1e4, rotary_dim=rotary, seed=91,
+                                                   scale=1.0, max_pos=2048)
+    common = common_blocks(page, False)
+    for turn, lengths in ((1, [170, 7]), (2, [33, 129, 1])):
+        specs = make_specs(common, lengths, turn, page, False)
+        *_, meta = run_prefill_parity(op, cpu_pool, dev_pool, specs, 1e4, gen, scale=1.0)
+        assert meta.launch.counts.kernel == 2 and meta.launch.counts.n_wide_items > 0
