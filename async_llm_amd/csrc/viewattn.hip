@@ -324,38 +324,43 @@ __global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// merge of partial states: one workgroup of 64 lanes per (row, q head)
+// merge of partial states: one workgroup of four waves per (row, q head)
 // ---------------------------------------------------------------------------
+// The launch is short and made of dependent loads (row list -> partial states), so it is laid out
+// for latency: wave w folds partials w, w + 4, ... of the row, eight per round with all their loads
+// in flight together, and the four running states meet in LDS.  Lane l owns dims l, l + 64, ...
+constexpr int kMergeWaves = 4;
+
 template <typename E>
-__global__ __launch_bounds__(64) void merge_kernel(MergeArgs a) {
+__global__ __launch_bounds__(64 * kMergeWaves) void merge_kernel(MergeArgs a) {
   using S = typename E::storage;
   const long long row = blockIdx.x;
   const int hq = blockIdx.y;
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
   const int flags = a.row_flags[row];
   if (flags & VA_ROW_DIRECT) return;
   S* o = (S*)a.out + (row * a.num_q_heads + hq) * (long long)a.head_dim;
   if (flags & VA_ROW_EMPTY) {
-    for (int d = threadIdx.x; d < a.head_dim; d += 64) o[d] = E::store(0.f);
+    for (int d = threadIdx.x; d < a.head_dim; d += 64 * kMergeWaves) o[d] = E::store(0.f);
     if (threadIdx.x == 0 && a.lse) a.lse[row * a.num_q_heads + hq] = -INFINITY;
     return;
   }
-  // One pass with a running (max, sum, accumulator); eight partials per round so
-  // that their loads are all in flight before the first one is folded in.
   const int b = a.row_indptr[row], e = a.row_indptr[row + 1];
-  const int n_d = (a.head_dim + 63) / 64;  // dims per thread: d = threadIdx.x + 64*k (at most 4 for D = 256)
+  const int n_d = (a.head_dim + 63) / 64;  // dims per lane: d = lane + 64*k (at most 4 for D = 256)
   float mm = kNegBig, ll = 0.f;
   float av[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int i0 = b; i0 < e; i0 += 8) {
+  for (int i0 = b + wave; i0 < e; i0 += 8 * kMergeWaves) {
     float mp[8], lp[8], ap[8][4];
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const int i = min(i0 + u, e - 1);
+      const int iu = i0 + u * kMergeWaves;
+      const int i = min(iu, e - 1);
       const long long slot = (long long)a.row_ids[i] * a.num_q_heads + hq;
-      mp[u] = i0 + u < e ? a.part_ml[slot * 2] : kNegBig;
-      lp[u] = i0 + u < e ? a.part_ml[slot * 2 + 1] : 0.f;
+      mp[u] = iu < e ? a.part_ml[slot * 2] : kNegBig;
+      lp[u] = iu < e ? a.part_ml[slot * 2 + 1] : 0.f;
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        const int d = threadIdx.x + 64 * k;
+        const int d = lane + 64 * k;
         ap[u][k] = (k < n_d && d < a.head_dim) ? a.part_acc[slot * a.head_dim + d] : 0.f;
       }
     }
@@ -369,12 +374,35 @@ __global__ __launch_bounds__(64) void merge_kernel(MergeArgs a) {
       mm = m_new;
     }
   }
+  // fold the waves' states: wave 0 collects
+  __shared__ float s_ml[kMergeWaves][2];
+  __shared__ float s_av[kMergeWaves][4][64];
+  if (wave > 0) {
+    if (lane == 0) {
+      s_ml[wave][0] = mm;
+      s_ml[wave][1] = ll;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) s_av[wave][k][lane] = av[k];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int w = 1; w < kMergeWaves; ++w) {
+    const float mw = s_ml[w][0], lw = s_ml[w][1];
+    const float m_new = fmaxf(mm, mw);
+    const float sa = exp2f(mm - m_new), sb = exp2f(mw - m_new);
+    ll = ll * sa + lw * sb;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) av[k] = av[k] * sa + s_av[w][k][lane] * sb;
+    mm = m_new;
+  }
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
-    const int d = threadIdx.x + 64 * k;
+    const int d = lane + 64 * k;
     if (d < a.head_dim) o[d] = E::store(ll > 0.f ? av[k] / ll : 0.f);
   }
-  if (threadIdx.x == 0 && a.lse) {
+  if (lane == 0 && a.lse) {
     const float lse2 = ll > 0.f ? mm + log2f(ll) : -INFINITY;
     a.lse[row * a.num_q_heads + hq] = a.lse_base2 ? lse2 : lse2 * kLn2;
   }
@@ -406,7 +434,7 @@ int launch_generic(const AttnArgs& a, int n_items, hipStream_t stream) {
 
 template <typename E>
 int launch_merge(const MergeArgs& a, int n_rows, hipStream_t stream) {
-  hipLaunchKernelGGL(merge_kernel<E>, dim3((unsigned)n_rows, (unsigned)a.num_q_heads), dim3(64), 0, stream, a);
+  hipLaunchKernelGGL(merge_kernel<E>, dim3((unsigned)n_rows, (unsigned)a.num_q_heads), dim3(64 * kMergeWaves), 0, stream, a);
   return check_hip(hipGetLastError(), "merge launch");
 }
 
