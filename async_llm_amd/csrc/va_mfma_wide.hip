@@ -33,7 +33,11 @@ namespace va {
 constexpr int kWideThreads = 256;
 constexpr int kWideWaves = 4;
 constexpr int kWideTokens = 32;  // tokens per K/V tile
-constexpr int kWideBuffers = 4;  // ring depth
+#ifndef VA_WIDE_BUFFERS
+#define VA_WIDE_BUFFERS 4
+#endif
+constexpr int kWideBuffers = VA_WIDE_BUFFERS;  // ring depth: kWideBuffers - 2 tiles in flight
+constexpr int kWideAhead = kWideBuffers - 2;    // a ring step requests the tile this far ahead
 
 template <int kD>
 struct WideShape {
@@ -203,9 +207,10 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
 
     // ---- set-up: first two tiles on their way, then the query tile (staged in buffers 2 and 3) ----
     __syncthreads();  // every wave is done with the previous link's buffers
-    if (0 < n_tiles) issue_now(0);
-    if (1 < n_tiles) issue_now(1);
-    va_u32x4* q_stage = (va_u32x4*)(lds + 2 * Sh::kBufferBytes);
+#pragma unroll
+    for (int i = 0; i < kWideAhead; ++i)
+      if (i < n_tiles) issue_now(i);
+    va_u32x4* q_stage = (va_u32x4*)(lds + kWideAhead * Sh::kBufferBytes);
     va_u32x4 qf[kB][kSteps];  // B operands: row of block b, dims [16s + 8h, +8)
 #pragma unroll
     for (int pass = 0; pass < kB; ++pass) {
@@ -262,16 +267,19 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     int next_step = 0;
     auto ring_step = [&]() __attribute__((always_inline)) {
       const int k = next_step++;
-      const bool refill = k + 2 < n_tiles;
+      const bool refill = k + kWideAhead < n_tiles;
       long long row = 0;  // looked up before the barrier: the latency hides behind the wait
-      if (refill && tile_is_plain(k + 2)) row = half_row(k + 2);
-      if (k + 1 < n_tiles) {
-        ring_barrier<kL>();  // only the loads of tile k + 1 may still be outstanding
+      if (refill && tile_is_plain(k + kWideAhead)) row = half_row(k + kWideAhead);
+      // only the loads of the tiles requested after tile k (up to kWideAhead - 1 of them) may still be outstanding
+      if (k + kWideAhead - 1 < n_tiles) {
+        ring_barrier<(kWideAhead - 1) * kL>();
+      } else if (kWideAhead > 2 && k + 1 < n_tiles) {
+        ring_barrier<kL>();
       } else {
         ring_barrier<0>();
       }
 #if VA_WIDE_EXPERIMENT != 5 && VA_WIDE_EXPERIMENT != 8  // 5, 8: computation only
-      if (refill) issue(k + 2, row);
+      if (refill) issue(k + kWideAhead, row);
 #endif
     };
 
