@@ -43,8 +43,7 @@ template <int kD>
 struct WideShape {
   static constexpr int kChunks = kD / 8;     // 16-byte pieces of a head row
   static constexpr int kSteps = kD / 16;     // contraction steps of K.Q^T (32x32x16)
-  static constexpr int kDimTiles = kD / 32;  // 32-dim tiles of the output = dims a lane owns per V token
-  static constexpr int kVDw = kD / 64;       // dwords of a V token a lane reads
+  static constexpr int kDimTiles = kD / 32;  // 32-dim tiles of the output
   static constexpr int kRowBytes = kChunks * 16;
   static constexpr int kRowsPerLoad = kWave / kChunks;              // tile rows one wave-level load covers
   static constexpr int kLoadsPerKind = kWideTokens / kRowsPerLoad;  // loads per K (or V) tile
@@ -68,6 +67,22 @@ __device__ __forceinline__ int wide_swz(int r) {
   return (r >> 1) & 7;
 }
 
+// V tiles are read with transposing loads (16 lanes fetch 4 tokens x 16 dims, 32 bytes per token):
+// moving token r's pieces by 2 (r % 4) puts the four rows of such a fetch side by side in one
+// 128-byte window.
+__device__ __forceinline__ int wide_vswz(int r) { return (r & 3) << 1; }
+
+// A transposing LDS read (ds_read_b64_tr_b16).  Within every group of 16 lanes, lane s supplies
+// the address of four 16-bit elements E[s][0..3]; lane i receives E[i / 4 + 4 k][i % 4], k = 0..3.
+// With lane s pointed at token T + s / 4, dims c + 4 (s % 4) .. + 3, lane i therefore receives
+// dim c + i of tokens T .. T + 3: four consecutive contraction elements of one row of V^T.
+__device__ __forceinline__ va_u32x2 lds_read_tr16(uint32_t lds_byte_address) {
+  typedef short v4s __attribute__((ext_vector_type(4)));
+  const v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) v4s*)(uintptr_t)lds_byte_address);
+  return __builtin_bit_cast(va_u32x2, r);
+}
+
 // max over the two half-waves (lanes l and l ^ 32) without touching LDS
 __device__ __forceinline__ float half_wave_max(float x) {
   const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
@@ -78,7 +93,7 @@ template <typename E, int kD>
 __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArgs a) {
   using S = typename E::storage;
   using Sh = WideShape<kD>;
-  constexpr int kChunks = Sh::kChunks, kSteps = Sh::kSteps, kDimTiles = Sh::kDimTiles, kVDw = Sh::kVDw;
+  constexpr int kChunks = Sh::kChunks, kSteps = Sh::kSteps, kDimTiles = Sh::kDimTiles;
   constexpr int kRowBytes = Sh::kRowBytes, kL = Sh::kLoadsPerWave, kB = Sh::kBlocks, kWaveRows = Sh::kWaveRows;
 
   extern __shared__ va_u32x4 smem[];
@@ -108,25 +123,34 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   const int p_shift = __builtin_ctz(P);  // t / P and t % P as shift and mask (power-of-two pages)
   const int row_bytes = (int)a.pool_row_stride * (int)sizeof(S);
 
-  // this lane's part of a wave-level load: row within the load and (swizzled) piece
+  // this lane's part of a wave-level load: row within the load and (swizzled) piece; waves 0 and 1
+  // load K halves, waves 2 and 3 V halves, each kind with its own swizzle
+  const bool wave_is_v = wave >= 2;
+  auto ld_swz = [&](int r) __attribute__((always_inline)) { return wave_is_v ? wide_vswz(r) : wide_swz<kD>(r); };
   const int ld_row0 = lane / kChunks;
-  const int ld_x0 = (lane % kChunks) ^ wide_swz<kD>(ld_row0);
+  const int ld_x0 = (lane % kChunks) ^ ld_swz(ld_row0);
   // byte offset, from the first row of its 16-token group, of what this lane fetches in load u of a
   // tile that lies entirely inside the visible range (uniform pages)
   uint32_t ld_off[kL];
 #pragma unroll
   for (int u = 0; u < kL; ++u)
-    ld_off[u] = (uint32_t)((u * Sh::kRowsPerLoad + ld_row0) * row_bytes + 16 * (ld_x0 ^ wide_swz<kD>(u * Sh::kRowsPerLoad)));
+    ld_off[u] = (uint32_t)((u * Sh::kRowsPerLoad + ld_row0) * row_bytes + 16 * (ld_x0 ^ ld_swz(u * Sh::kRowsPerLoad)));
   // LDS offsets of what this lane reads from a tile
   const int swz_j = wide_swz<kD>(j);
   const int k_row_byte = j * kRowBytes;
-  int v_byte[8];  // token e of a 16-token step: (e / 4) * 8 + 4h + e % 4
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int tok = (e / 4) * 8 + 4 * h + (e % 4);
-    const int first_dim = j * (kD / 32);  // the lane's run of D/32 dims
-    v_byte[e] = tok * kRowBytes + 16 * ((first_dim / 8) ^ wide_swz<kD>(tok)) + 2 * (first_dim % 8);
-  }
+  // V^T fragments come from transposing reads.  For dim tile t (dims 32t .. 32t+31) and 16-token
+  // step kk the lane needs, as contraction elements 0..3 and 4..7, tokens 16kk + 4h + 0..3 and
+  // 16kk + 8 + 4h + 0..3 of dim 32t + lane % 32 (the token order P^T has in its registers): two
+  // reads, in each of which this lane points at token row `v_row` (+ 16kk, + 8) and at 4 dims of
+  // the tile's 16-dim half lane / 16 % 2.  The swizzle folds into two per-lane bases, one for even
+  // and one for odd t; everything else is an immediate offset.
+  const int v_sub = lane % 16;
+  const int v_row = 4 * h + v_sub / 4;
+  const int v_swz = wide_vswz(v_row);
+  const int v_piece = (2 * ((lane / 16) % 2) + (v_sub % 4) / 2) ^ (v_swz & 2);
+  const int v_base = v_row * kRowBytes + 16 * v_piece + 8 * (v_sub % 2);
+  const int v_even = v_base + 64 * (v_swz >> 2), v_odd = v_base + 64 * (1 ^ (v_swz >> 2));
+  const uint32_t lds_base = lds_address(lds);
 
   float m_ref[kB], m_tile[kB], l_run[kB];  // reference maximum (log2 units), last tile maximum, row sum
   va_f32x16 o[kB][kDimTiles];
@@ -171,7 +195,6 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     // the visible range, and page tables with pages under 16 tokens or slot lists, look every
     // row up per lane instead (rows past the range re-read the last visible token; their scores
     // are masked).
-    const bool wave_is_v = wave >= 2;
     const int wave_half = wave & 1;
     const char* wave_pool = (const char*)(wave_is_v ? vp : kp);
     const uint32_t wave_lds = __builtin_amdgcn_readfirstlane(lds_address(lds)) + (wave_is_v ? Sh::kTileBytes : 0) +
@@ -198,7 +221,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         for (int u = 0; u < kL; ++u) {
           const int r = u * Sh::kRowsPerLoad + ld_row0;
           const int t = min(t0 + r, t_last);
-          const int piece = 16 * (ld_x0 ^ wide_swz<kD>(u * Sh::kRowsPerLoad));
+          const int piece = 16 * (ld_x0 ^ ld_swz(u * Sh::kRowsPerLoad));
           load_to_lds(wave_pool + kv_slot(a.kv_indices, kv_begin, t, P, slots) * row_bytes + piece, dst + u * 1024);
         }
       }
@@ -278,7 +301,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       } else {
         ring_barrier<0>();
       }
-#if VA_WIDE_EXPERIMENT != 5 && VA_WIDE_EXPERIMENT != 8  // 5, 8: computation only
+#if VA_WIDE_EXPERIMENT != 5  // 5: computation only
       if (refill) issue(k + kWideAhead, row);
 #endif
     };
@@ -288,12 +311,6 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     va_u32x4 kf[kSteps];
     auto read_k = [&](int tile) __attribute__((always_inline)) {
       const char* kt = lds + (tile % kWideBuffers) * Sh::kBufferBytes;
-#if VA_WIDE_EXPERIMENT == 8  // no LDS reads: one fragment stands in for all
-      kf[0] = *(const va_u32x4*)(kt + k_row_byte);
-#pragma unroll
-      for (int s = 1; s < kSteps; ++s) kf[s] = kf[0] + (uint32_t)s;
-      return;
-#endif
 #pragma unroll
       for (int s = 0; s < kSteps; ++s) kf[s] = *(const va_u32x4*)(kt + k_row_byte + 16 * ((2 * s + h) ^ swz_j));
     };
@@ -349,26 +366,17 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         }
         resume = false;
 
-        const char* vt = lds + (i % kWideBuffers) * Sh::kBufferBytes + Sh::kTileBytes;
-        uint32_t vraw[2][8][kVDw];
-        auto read_v = [&](int kk) __attribute__((always_inline)) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-#if VA_WIDE_EXPERIMENT == 8
-            const char* at = vt + v_byte[0];
-#else
-            const char* at = vt + v_byte[e] + kk * 16 * kRowBytes;
-#endif
-            if constexpr (kVDw == 4) {
-              const va_u32x4 x = *(const va_u32x4*)at;
-              vraw[kk][e][0] = x[0]; vraw[kk][e][1] = x[1]; vraw[kk][e][2] = x[2]; vraw[kk][e][3] = x[3];
-            } else if constexpr (kVDw == 2) {
-              const uint2 x = *(const uint2*)at;
-              vraw[kk][e][0] = x.x; vraw[kk][e][1] = x.y;
-            } else {
-              vraw[kk][e][0] = *(const uint32_t*)at;
-            }
-          }
+        // V^T fragments of this tile, kVAhead of them in flight: fragment idx = (step kk, dim tile t)
+        const uint32_t vt = lds_base + (i % kWideBuffers) * Sh::kBufferBytes + Sh::kTileBytes;
+        const uint32_t vt_even = vt + v_even, vt_odd = vt + v_odd;
+        constexpr int kFrags = 2 * kDimTiles;
+        constexpr int kVAhead = kFrags < 4 ? kFrags : 4;
+        va_u32x4 vfr[kVAhead];
+        auto read_vfrag = [&](int idx) __attribute__((always_inline)) {
+          const int kk = idx / kDimTiles, t = idx % kDimTiles;
+          const uint32_t at = ((t & 1) ? vt_odd : vt_even) + 128 * (t / 2) + kk * 16 * kRowBytes;
+          const va_u32x2 lo = lds_read_tr16(at), hi = lds_read_tr16(at + 8 * kRowBytes);
+          vfr[idx % kVAhead] = va_u32x4{lo[0], lo[1], hi[0], hi[1]};
         };
         // ---- phase A: scores of tile i + 1 (matrix pipe) under the exponentials of tile i ----
         float sum[kB];
@@ -388,7 +396,8 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         constexpr int kPiecesPerStep = 16 / kSteps > 0 ? 16 / kSteps : 1;  // exponentials between two score steps
         if (has_next) {
           read_k(i + 1);
-          read_v(0);
+#pragma unroll
+          for (int idx = 0; idx < kVAhead; ++idx) read_vfrag(idx);
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
@@ -398,7 +407,8 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
             __builtin_amdgcn_sched_barrier(0);
           }
         } else {
-          read_v(0);
+#pragma unroll
+          for (int idx = 0; idx < kVAhead; ++idx) read_vfrag(idx);
 #pragma unroll
           for (int r = 0; r < 16; ++r) exp_piece(r);
         }
@@ -408,31 +418,22 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
           pw[b][7] = Mma<E>::pack(sc[b][14], sc[b][15]);
         }
 
-        // ---- phase B: O^T += V^T . P^T over two 16-token steps; while a product runs, the V
-        // fragment of the next one is transposed; a transposed fragment serves all row blocks ----
-        read_v(1);
+        // ---- phase B: O^T += V^T . P^T over two 16-token steps; a fragment serves all row blocks,
+        // and once it has been used the fragment kVAhead further on is requested ----
         va_u32x4 pf[2][kB];
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
           for (int b = 0; b < kB; ++b)
             pf[kk][b] = va_u32x4{pw[b][4 * kk + 0], pw[b][4 * kk + 1], pw[b][4 * kk + 2], pw[b][4 * kk + 3]};
-        auto transposed = [&](int idx) __attribute__((always_inline)) {
-          const int kk = idx / kDimTiles, t = idx % kDimTiles;
-          const int w = t / 2;
-          const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
-          return va_u32x4{__builtin_amdgcn_perm(vraw[kk][1][w], vraw[kk][0][w], sel), __builtin_amdgcn_perm(vraw[kk][3][w], vraw[kk][2][w], sel),
-                          __builtin_amdgcn_perm(vraw[kk][5][w], vraw[kk][4][w], sel), __builtin_amdgcn_perm(vraw[kk][7][w], vraw[kk][6][w], sel)};
-        };
-        va_u32x4 vf = transposed(0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int idx = 0; idx < 2 * kDimTiles; ++idx) {
+        for (int idx = 0; idx < kFrags; ++idx) {
           const int kk = idx / kDimTiles, t = idx % kDimTiles;
 #pragma unroll
-          for (int b = 0; b < kB; ++b) Mma<E>::run32_acc(vf, pf[kk][b], o[b][t]);
+          for (int b = 0; b < kB; ++b) Mma<E>::run32_acc(vfr[idx % kVAhead], pf[kk][b], o[b][t]);
           __builtin_amdgcn_sched_barrier(0);
-          if (idx + 1 < 2 * kDimTiles) vf = transposed(idx + 1);
+          if (idx + kVAhead < kFrags) read_vfrag(idx + kVAhead);
           __builtin_amdgcn_sched_barrier(0);
         }
         if (has_next) {  // the scores of tile i + 1 were complete long before the last product
@@ -458,7 +459,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   }
 
   accumulator_fence();
-  // ---- emit: accumulator reg r of dim tile T is dim ((r/4)*8 + 4h + r%4) * D/32 + T of the lane's row ----
+  // ---- emit: accumulator reg r of dim tile t is dim 32t + (r/4)*8 + 4h + r%4 of the lane's row ----
 #pragma unroll
   for (int b = 0; b < kB; ++b) {
     float l = l_run[b];
@@ -478,19 +479,13 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       const long long out_row = a.sub_worker[subrow];
       S* orow = (S*)a.out + (out_row * a.num_q_heads + hq) * (long long)kD;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int d0 = ((r / 4) * 8 + 4 * h + (r % 4)) * kDimTiles;
-        uint32_t w[kDimTiles / 2];
+      for (int t = 0; t < kDimTiles; ++t)
 #pragma unroll
-        for (int t = 0; t < kDimTiles / 2; ++t) w[t] = Mma<E>::pack(o[b][2 * t][r] * inv, o[b][2 * t + 1][r] * inv);
-        if constexpr (kDimTiles == 8) {
-          *(uint4*)(orow + d0) = make_uint4(w[0], w[1], w[2], w[3]);
-        } else if constexpr (kDimTiles == 4) {
-          *(uint2*)(orow + d0) = make_uint2(w[0], w[1]);
-        } else {
-          *(uint32_t*)(orow + d0) = w[0];
+        for (int r = 0; r < 16; r += 4) {  // four consecutive dims
+          const int d0 = 32 * t + (r / 4) * 8 + 4 * h;
+          *(uint2*)(orow + d0) = make_uint2(Mma<E>::pack(o[b][t][r] * inv, o[b][t][r + 1] * inv),
+                                            Mma<E>::pack(o[b][t][r + 2] * inv, o[b][t][r + 3] * inv));
         }
-      }
       if (h == 0 && a.lse) {
         const float lse2 = l > 0.f ? m_ref[b] + log2f(l) : -INFINITY;
         a.lse[out_row * a.num_q_heads + hq] = a.lse_base2 ? lse2 : lse2 * kLn2;
@@ -499,11 +494,10 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       const long long slot = (long long)(part_base + iq) * a.num_q_heads + hq;
       float* prow = a.part_acc + slot * kD;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int d0 = ((r / 4) * 8 + 4 * h + (r % 4)) * kDimTiles;
+      for (int t = 0; t < kDimTiles; ++t)
 #pragma unroll
-        for (int t = 0; t < kDimTiles; ++t) prow[d0 + t] = o[b][t][r];
-      }
+        for (int r = 0; r < 16; r += 4)
+          *(float4*)(prow + 32 * t + (r / 4) * 8 + 4 * h) = make_float4(o[b][t][r], o[b][t][r + 1], o[b][t][r + 2], o[b][t][r + 3]);
       if (h == 0) {
         a.part_ml[slot * 2 + 0] = m_ref[b];
         a.part_ml[slot * 2 + 1] = l;
