@@ -335,6 +335,12 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       for (int b = 0; b < kB; ++b) sc[b] = sc_next[b];
     }
     bool resume = false;  // the step for tile i + 1 is made and sc holds the (masked) scores of tile i
+    // maximum of the (unmasked) scores of the next tile per lane, gathered piecewise between the
+    // P.V products of the current one, whose matrix work leaves the vector ALU idle
+    float early_max[kB];
+    bool early_max_valid = false;
+#pragma unroll
+    for (int b = 0; b < kB; ++b) early_max[b] = 0.f;
     int i = 0;
     while (i < n_vis) {
       for (; i < n_vis; ++i) {
@@ -352,9 +358,12 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
               for (int r = 0; r < 16; ++r)
                 sc[b][r] = (t0 + (r / 4) * 8 + 4 * h + (r % 4)) < t_row[b] ? sc[b][r] : -INFINITY;
             }
-            float tile_max = sc[b][0];
+            float tile_max = early_max[b];  // found under the previous tile's P.V products
+            if (masked || !early_max_valid) {
+              tile_max = sc[b][0];
 #pragma unroll
-            for (int r = 1; r < 16; ++r) tile_max = fmaxf(tile_max, sc[b][r]);
+              for (int r = 1; r < 16; ++r) tile_max = fmaxf(tile_max, sc[b][r]);
+            }
             tile_max = half_wave_max(tile_max);
             m_tile[b] = tile_max * a.scale_log2;
             raise = raise || m_tile[b] > m_ref[b] + kRaise;
@@ -370,6 +379,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         const uint32_t vt = lds_base + (i % kWideBuffers) * Sh::kBufferBytes + Sh::kTileBytes;
         const uint32_t vt_even = vt + v_even, vt_odd = vt + v_odd;
         constexpr int kFrags = 2 * kDimTiles;
+        constexpr int kMaxFirst = kFrags > 2 ? 2 : kFrags - 1;  // first product the early maxima follow
         constexpr int kVAhead = kFrags < 4 ? kFrags : 4;
         va_u32x4 vfr[kVAhead];
         auto read_vfrag = [&](int idx) __attribute__((always_inline)) {
@@ -434,8 +444,21 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
           for (int b = 0; b < kB; ++b) Mma<E>::run32_acc(vfr[idx % kVAhead], pf[kk][b], o[b][t]);
           __builtin_amdgcn_sched_barrier(0);
           if (idx + kVAhead < kFrags) read_vfrag(idx + kVAhead);
+          // Elements of the next tile's scores folded into early_max after this product: the 15
+          // comparisons are spread over the products from the third on (the last score product was
+          // issued well before, so its results have been written).
+          if (idx >= kMaxFirst) {
+#pragma unroll
+            for (int e = 1; e < 16; ++e) {
+              if (kMaxFirst + (e - 1) * (kFrags - kMaxFirst) / 15 != idx) continue;
+#pragma unroll
+              for (int b = 0; b < kB; ++b)
+                early_max[b] = fmaxf(e == 1 ? sc_next[b][0] : early_max[b], sc_next[b][e]);
+            }
+          }
           __builtin_amdgcn_sched_barrier(0);
         }
+        early_max_valid = has_next;
         if (has_next) {  // the scores of tile i + 1 were complete long before the last product
 #pragma unroll
           for (int b = 0; b < kB; ++b) sc[b] = sc_next[b];
