@@ -35,6 +35,11 @@ struct Mma<BF16> {
   static __device__ __forceinline__ void run32_acc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
+  // ... without the wait states: for products whose operands no vector-ALU instruction has written
+  // since an earlier product of the same run was issued
+  static __device__ __forceinline__ void run32_acc_next(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
   // The same with the accumulator in ordinary vector registers (for results the vector ALU reads
   // next, the scores); `first`: the sum starts from zero.  No leading s_nop: the operands of these
   // products come from LDS reads and from registers written long before.
@@ -54,9 +59,11 @@ struct Mma<BF16> {
     return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(va_i16x4, a), __builtin_bit_cast(va_i16x4, b),
                                                      c, 0, 0, 0);
   }
+  // both conversions in one instruction (v_cvt_pk_bf16_f32, round to nearest even)
   static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    const __bf16 l = (__bf16)lo, h = (__bf16)hi;
-    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
   }
 };
 template <>
@@ -68,6 +75,9 @@ struct Mma<F16> {
   }
   static __device__ __forceinline__ void run32_acc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void run32_acc_next(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ void run32_vacc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
@@ -85,8 +95,9 @@ struct Mma<F16> {
                                                  0, 0, 0);
   }
   static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    const _Float16 l = (_Float16)lo, h = (_Float16)hi;
-    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, f16x2));
   }
 };
 

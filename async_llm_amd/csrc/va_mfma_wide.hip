@@ -288,11 +288,17 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     const int n_vis = t_wave > tok_begin ? min(n_tiles, (t_wave - tok_begin + kWideTokens - 1) / kWideTokens) : 0;
 #endif
     int next_step = 0;
+    // The pool row of the tile a step requests is looked up a whole step earlier (a scalar load whose
+    // result is not touched before the next step): its latency never shows.
+    auto row_of = [&](int tile) __attribute__((always_inline)) {
+      return (tile < n_tiles && tile_is_plain(tile)) ? half_row(tile) : 0ll;
+    };
+    long long row_ahead = row_of(kWideAhead);
     auto ring_step = [&]() __attribute__((always_inline)) {
       const int k = next_step++;
       const bool refill = k + kWideAhead < n_tiles;
-      long long row = 0;  // looked up before the barrier: the latency hides behind the wait
-      if (refill && tile_is_plain(k + kWideAhead)) row = half_row(k + kWideAhead);
+      const long long row = row_ahead;
+      row_ahead = row_of(k + 1 + kWideAhead);
       // only the loads of the tiles requested after tile k (up to kWideAhead - 1 of them) may still be outstanding
       if (k + kWideAhead - 1 < n_tiles) {
         ring_barrier<(kWideAhead - 1) * kL>();
@@ -441,7 +447,14 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         for (int idx = 0; idx < kFrags; ++idx) {
           const int kk = idx / kDimTiles, t = idx % kDimTiles;
 #pragma unroll
-          for (int b = 0; b < kB; ++b) Mma<E>::run32_acc(vfr[idx % kVAhead], pf[kk][b], o[b][t]);
+          for (int b = 0; b < kB; ++b) {
+            // P was packed by the vector ALU just before the first product; V fragments come from LDS
+            if (idx == 0) {
+              Mma<E>::run32_acc(vfr[idx % kVAhead], pf[kk][b], o[b][t]);
+            } else {
+              Mma<E>::run32_acc_next(vfr[idx % kVAhead], pf[kk][b], o[b][t]);
+            }
+          }
           __builtin_amdgcn_sched_barrier(0);
           if (idx + kVAhead < kFrags) read_vfrag(idx + kVAhead);
           // Elements of the next tile's scores folded into early_max after this product: the 15
