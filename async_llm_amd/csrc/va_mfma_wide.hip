@@ -341,6 +341,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       for (int b = 0; b < kB; ++b) sc[b] = sc_next[b];
     }
     bool resume = false;  // the step for tile i + 1 is made and sc holds the (masked) scores of tile i
+    bool sc_is_raw = true;  // sc holds the raw scores of the first tile (no reference maximum exists yet)
     // maximum of the (unmasked) scores of the next tile per lane, gathered piecewise between the
     // P.V products of the current one, whose matrix work leaves the vector ALU idle
     float early_max[kB];
@@ -364,17 +365,19 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
               for (int r = 0; r < 16; ++r)
                 sc[b][r] = (t0 + (r / 4) * 8 + 4 * h + (r % 4)) < t_row[b] ? sc[b][r] : -INFINITY;
             }
-            float tile_max = early_max[b];  // found under the previous tile's P.V products
+            // the tile maximum in log2 units: from the raw maxima found under the previous products, or,
+            // for a masked or first tile, from sc (raw scores on the first tile, else already s - m_ref)
+            float tile_max = early_max[b] * a.scale_log2;
             if (masked || !early_max_valid) {
               tile_max = sc[b][0];
 #pragma unroll
               for (int r = 1; r < 16; ++r) tile_max = fmaxf(tile_max, sc[b][r]);
+              tile_max = sc_is_raw ? tile_max * a.scale_log2 : tile_max + m_ref[b];
             }
-            tile_max = half_wave_max(tile_max);
-            m_tile[b] = tile_max * a.scale_log2;
+            m_tile[b] = half_wave_max(tile_max);
             raise = raise || m_tile[b] > m_ref[b] + kRaise;
           }
-          if (__any(raise)) {
+          if (__any(raise) || sc_is_raw) {  // the first tile always sets the references
             resume = true;
             break;
           }
@@ -404,7 +407,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         auto exp_piece = [&](int r) __attribute__((always_inline)) {
 #pragma unroll
           for (int b = 0; b < kB; ++b) {
-            sc[b][r] = __builtin_amdgcn_exp2f(fmaf(sc[b][r], a.scale_log2, -m_ref[b]));
+            sc[b][r] = __builtin_amdgcn_exp2f(sc[b][r]);  // sc holds s - m_ref already
             if (r > 0) sum[b] += sc[b][r - 1];
             if (r >= 2 && r % 2 == 0) pw[b][r / 2 - 1] = Mma<E>::pack(sc[b][r - 2], sc[b][r - 1]);
           }
@@ -468,14 +471,18 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
               for (int b = 0; b < kB; ++b)
                 early_max[b] = fmaxf(e == 1 ? sc_next[b][0] : early_max[b], sc_next[b][e]);
             }
+            // ... and moved to sc as s * scale - m_ref, what the exponentials of the next iteration
+            // start from (P of this tile has left sc; a raised reference redoes this from sc_next)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+              if (kMaxFirst + e * (kFrags - kMaxFirst) / 16 != idx) continue;
+#pragma unroll
+              for (int b = 0; b < kB; ++b) sc[b][e] = fmaf(sc_next[b][e], a.scale_log2, -m_ref[b]);
+            }
           }
           __builtin_amdgcn_sched_barrier(0);
         }
         early_max_valid = has_next;
-        if (has_next) {  // the scores of tile i + 1 were complete long before the last product
-#pragma unroll
-          for (int b = 0; b < kB; ++b) sc[b] = sc_next[b];
-        }
       }
       if (resume) {
         // raise the references to this tile's maxima and rescale what was accumulated against the old ones
@@ -488,7 +495,15 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
           l_run[b] *= alpha;
 #pragma unroll
           for (int t = 0; t < kDimTiles; ++t) o[b][t] *= alpha;
+          // sc_next still holds this tile's raw scores: sc = s * scale - m_ref against the new reference
+          const int t0 = tok_begin + i * kWideTokens;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const bool visible = (t0 + (r / 4) * 8 + 4 * h + (r % 4)) < t_row[b];
+            sc[b][r] = visible ? fmaf(sc_next[b][r], a.scale_log2, -m_ref[b]) : -INFINITY;
+          }
         }
+        sc_is_raw = false;
       }
     }
     while (next_step < n_tiles) ring_step();  // tiles this wave does not see: keep in step with the others
