@@ -186,6 +186,14 @@ template <int n>
 __device__ __forceinline__ void ring_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(n) : "memory");
 }
+// The same, handing back a zero that exists only after the barrier: a value combined with it cannot
+// be touched (and so cannot be waited for) before the barrier.
+template <int n>
+__device__ __forceinline__ int ring_barrier_zero() {
+  int zero;
+  asm volatile("s_waitcnt vmcnt(%1) lgkmcnt(0)\n\ts_barrier\n\ts_mov_b32 %0, 0" : "=s"(zero) : "n"(n) : "memory");
+  return zero;
+}
 constexpr int kAnyInFlight = 63;  // vmcnt(63): no wait on vector memory at all
 
 // One wave-level pool -> LDS load: lane l's 16 bytes at `src` land at LDS byte address

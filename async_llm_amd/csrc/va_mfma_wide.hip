@@ -312,6 +312,30 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
 #endif
     };
 
+    // The same step for the steady part of a link (uniform pages; the requested tile and the one
+    // after it inside the visible range): no case distinctions, and the page lookup for the next
+    // step is sent before the barrier and first touched after it, so its latency passes under the wait.
+    auto ring_step_steady = [&]() __attribute__((always_inline)) {
+      const int k = next_step++;
+      const long long row = row_ahead;
+      const int t = tok_begin + (k + 1 + kWideAhead) * kWideTokens + 16 * wave_half;
+      const int page = ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + (t >> p_shift)];
+      const int zero = ring_barrier_zero<(kWideAhead - 1) * kL>();
+      const uint32_t dst = wave_lds + ((k + kWideAhead) % kWideBuffers) * Sh::kBufferBytes;
+      const char* base = wave_pool + row * row_bytes;
+#pragma unroll
+      for (int u = 0; u < kL; ++u) load_to_lds(base, ld_off[u], dst + u * 1024);
+      row_ahead = ((long long)(page + zero) << p_shift) + (t & (P - 1));
+    };
+    // iterations [1, i_steady_end) may take it: tiles i + 1 + kWideAhead and i + 2 + kWideAhead are plain,
+    // tile i is unmasked for every row of the wave and a next tile exists
+    int i_steady_end = 0;
+    if (uniform_pages) {
+      const int plain_tiles = (t_last + 1 - tok_begin) / kWideTokens;  // tiles 0 .. plain_tiles - 1 are plain
+      const int unmasked_tiles = t_wave_min > tok_begin ? (t_wave_min - tok_begin) / kWideTokens : 0;
+      i_steady_end = min(min(plain_tiles - 2 - kWideAhead, unmasked_tiles), n_vis - 1);
+    }
+
     va_f32x16 sc[kB];       // scores, then probabilities, of the current tile
     va_f32x16 sc_next[kB];  // scores of the next tile, accumulating
     va_u32x4 kf[kSteps];
@@ -353,7 +377,20 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       for (; i < n_vis; ++i) {
         const int t0 = tok_begin + i * kWideTokens;
         const bool has_next = i + 1 < n_vis;
-        if (!resume) {
+        if (!resume && i >= 1 && i < i_steady_end) {
+          // steady part: the maxima were gathered under the previous products, nothing is masked
+          ring_step_steady();
+          bool raise = false;
+#pragma unroll
+          for (int b = 0; b < kB; ++b) {
+            m_tile[b] = half_wave_max(early_max[b] * a.scale_log2);
+            raise = raise || m_tile[b] > m_ref[b] + kRaise;
+          }
+          if (__any(raise)) {
+            resume = true;
+            break;
+          }
+        } else if (!resume) {
           if (i + 1 < n_tiles) ring_step();  // tile i + 1 has landed
           // mask and find the tile maxima; reg r of a block is token t0 + (r/4)*8 + 4h + r%4 of its row
           const bool masked = t0 + kWideTokens > t_wave_min;
