@@ -444,29 +444,27 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         auto exp_piece = [&](int r) __attribute__((always_inline)) {
 #pragma unroll
           for (int b = 0; b < kB; ++b) {
-            sc[b][r] = __builtin_amdgcn_exp2f(sc[b][r]);  // sc holds s - m_ref already
+            // sc holds s - m_ref already; issued from assembly so that it stays where it is written,
+            // between two score products
+            asm volatile("v_exp_f32 %0, %0" : "+v"(sc[b][r]));
             if (r > 0) sum[b] += sc[b][r - 1];
             if (r >= 2 && r % 2 == 0) pw[b][r / 2 - 1] = Mma<E>::pack(sc[b][r - 2], sc[b][r - 1]);
           }
         };
         constexpr int kPiecesPerStep = 16 / kSteps > 0 ? 16 / kSteps : 1;  // exponentials between two score steps
-        if (has_next) {
-          read_k(i + 1);
+        // The last visible tile runs the same instructions: its "next scores" come from whatever
+        // the following ring buffer holds and are never looked at (sixteen idle products per link
+        // against a second copy of this phase and the register moves where the two would meet).
+        read_k(i + 1);
 #pragma unroll
-          for (int idx = 0; idx < kVAhead; ++idx) read_vfrag(idx);
+        for (int idx = 0; idx < kVAhead; ++idx) read_vfrag(idx);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          if (r % kPiecesPerStep == 0) score_step(r / kPiecesPerStep);
           __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            if (r % kPiecesPerStep == 0) score_step(r / kPiecesPerStep);
-            __builtin_amdgcn_sched_barrier(0);
-            exp_piece(r);
-            __builtin_amdgcn_sched_barrier(0);
-          }
-        } else {
-#pragma unroll
-          for (int idx = 0; idx < kVAhead; ++idx) read_vfrag(idx);
-#pragma unroll
-          for (int r = 0; r < 16; ++r) exp_piece(r);
+          exp_piece(r);
+          __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int b = 0; b < kB; ++b) {
