@@ -173,6 +173,54 @@ __device__ __forceinline__ void rotated_query_unit(const RopeDev& rope, const ty
   o1 = make_uint4(hi[0], hi[1], hi[2], hi[3]);
 }
 
+// The same unit in two steps for the cos|sin table, for callers that stage several rows at once:
+// `load` sends every memory request of the unit (the two query pieces and the sixteen table
+// entries), `finish` rotates.  A caller that loads a batch of rows before it finishes the first
+// pays the memory latency once per batch instead of once per row.  The unit must be rotary
+// (x < rotary_dim / 16); pieces past the rotary part are plain copies.
+template <typename E>
+struct TableQueryUnit {
+  uint4 ra, rb;
+  float4 c[2], s[2];
+  __device__ __forceinline__ void load(const RopeDev& rope, const typename E::storage* qh, int x, const Pos3& p) {
+    const int i0 = 8 * x;
+    ra = *(const uint4*)(qh + i0);
+    rb = *(const uint4*)(qh + i0 + rope.half);
+    long long a = p.t < 0 ? -p.t : p.t;
+    if (a > rope.max_pos - 1) a = rope.max_pos - 1;
+    // rows of the table and their halves start on 32-byte boundaries (rotary_dim is a multiple of 16)
+    const float* row = rope.cos_sin + a * (long long)rope.rotary_dim + i0;
+    c[0] = *(const float4*)row;
+    c[1] = *(const float4*)(row + 4);
+    s[0] = *(const float4*)(row + rope.half);
+    s[1] = *(const float4*)(row + rope.half + 4);
+  }
+  __device__ __forceinline__ void finish(const RopeDev& rope, const Pos3& p, uint4& o0, uint4& o1) const {
+    using S = typename E::storage;
+    const uint32_t wa[4] = {ra.x, ra.y, ra.z, ra.w}, wb[4] = {rb.x, rb.y, rb.z, rb.w};
+    const float ct[8] = {c[0].x, c[0].y, c[0].z, c[0].w, c[1].x, c[1].y, c[1].z, c[1].w};
+    const float st[8] = {s[0].x, s[0].y, s[0].z, s[0].w, s[1].x, s[1].y, s[1].z, s[1].w};
+    uint32_t lo[4], hi[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      float y1[2], y2[2];
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const S xa = __builtin_bit_cast(S, (uint16_t)(wa[w] >> (16 * b)));
+        const S xb = __builtin_bit_cast(S, (uint16_t)(wb[w] >> (16 * b)));
+        const float sn = p.t < 0 ? -st[2 * w + b] : st[2 * w + b];
+        // the table mode's arithmetic of rope_pair: fp32, one rounding at the end
+        y1[b] = round_through<E>(mul_rounded(ct[2 * w + b], E::load(xa)) - mul_rounded(sn, E::load(xb)));
+        y2[b] = round_through<E>(mul_rounded(ct[2 * w + b], E::load(xb)) + mul_rounded(sn, E::load(xa)));
+      }
+      lo[w] = Mma<E>::pack(y1[0], y1[1]);  // already representable: the conversions are exact
+      hi[w] = Mma<E>::pack(y2[0], y2[1]);
+    }
+    o0 = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    o1 = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+  }
+};
+
 // Wait until the matrix pipe has written the results of products issued from assembly
 // (run32_acc): 8 passes plus the write-back, 20 wait states.
 __device__ __forceinline__ void accumulator_fence() { asm volatile("s_nop 15\n\ts_nop 3" ::: "memory"); }

@@ -237,21 +237,84 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     va_u32x4 qf[kB][kSteps];  // B operands: row of block b, dims [16s + 8h, +8)
 #pragma unroll
     for (int pass = 0; pass < kB; ++pass) {
-      for (int idx = tid; idx < 128 * (kChunks / 2); idx += kWideThreads) {  // two pieces per step
-        const int Rl = idx / (kChunks / 2), x = idx - Rl * (kChunks / 2);
-        const int R = kWaveRows * (Rl / 32) + 32 * pass + Rl % 32;  // block `pass` of every wave
-        const int iq = R / G, g = R - iq * G;
-        int c0 = 2 * x, c1 = 2 * x + 1;
-        uint4 p0 = make_uint4(0, 0, 0, 0), p1 = p0;
-        if (iq < n_q) {
-          const int subrow = (lflags & VA_LINK_INDIRECT) ? a.qrefs[qref + iq] : qref + iq;
-          const long long src_row = a.sub_worker[subrow];
-          const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
-          const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
-          rotated_query_unit<E>(a.rope, qh, x, p, c0, c1, p0, p1);
+      if (a.rope.mode == VA_ROPE_TABLE) {
+        // Every thread stages one unit (two pieces) of kIts rows.  The sub-row numbers are fetched
+        // for all rows at once, source rows and positions, then pieces and table entries, for
+        // kBatch rows at once: a row's chain of dependent loads (sub-row -> source row and position
+        // -> query pieces and cos|sin entries) is paid once per batch, not once per row (row by row
+        // this set-up was an eighth of the kernel on long views of many blocks).
+        constexpr int kUnits = kChunks / 2, kRowStep = kWideThreads / kUnits, kIts = 128 / kRowStep;
+        constexpr int kBatch = kIts < 2 ? kIts : 2;
+        static_assert(kWideThreads % kUnits == 0 && 128 % kRowStep == 0 && kIts % kBatch == 0, "staging pattern");
+        const int x = tid % kUnits, rl0 = tid / kUnits;
+        const int pair_units = a.rope.rotary_dim / 16;
+        const bool rotary = x < pair_units;
+        const int c0 = rotary ? x : a.rope.rotary_dim / 8 + 2 * (x - pair_units);
+        const int c1 = rotary ? x + pair_units : c0 + 1;
+        bool live[kIts];
+        int subrow[kIts];
+#pragma unroll
+        for (int it = 0; it < kIts; ++it) {
+          const int Rl = rl0 + it * kRowStep;
+          const int R = kWaveRows * (Rl / 32) + 32 * pass + Rl % 32;  // block `pass` of every wave
+          const int iq = R / G;
+          live[it] = iq < n_q;
+          const int iqc = live[it] ? iq : 0;  // rows past the tile stage row 0's numbers and are zeroed below
+          subrow[it] = (lflags & VA_LINK_INDIRECT) ? a.qrefs[qref + iqc] : qref + iqc;
         }
-        q_stage[Rl * kChunks + (c0 ^ wide_swz<kD>(Rl))] = va_u32x4{p0.x, p0.y, p0.z, p0.w};
-        q_stage[Rl * kChunks + (c1 ^ wide_swz<kD>(Rl))] = va_u32x4{p1.x, p1.y, p1.z, p1.w};
+#pragma unroll
+        for (int it0 = 0; it0 < kIts; it0 += kBatch) {
+          const S* qh[kBatch];
+          Pos3 pos[kBatch];
+#pragma unroll
+          for (int jj = 0; jj < kBatch; ++jj) {
+            const int Rl = rl0 + (it0 + jj) * kRowStep;
+            const int R = kWaveRows * (Rl / 32) + 32 * pass + Rl % 32;
+            const int iq = R / G, g = R - iq * G;
+            const long long src_row = a.sub_worker[subrow[it0 + jj]];
+            qh[jj] = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
+            pos[jj] = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow[it0 + jj]);
+          }
+          uint4 p0[kBatch], p1[kBatch];
+          if (rotary) {
+            TableQueryUnit<E> unit[kBatch];
+#pragma unroll
+            for (int jj = 0; jj < kBatch; ++jj) unit[jj].load(a.rope, qh[jj], x, pos[jj]);
+#pragma unroll
+            for (int jj = 0; jj < kBatch; ++jj) unit[jj].finish(a.rope, pos[jj], p0[jj], p1[jj]);
+          } else {
+#pragma unroll
+            for (int jj = 0; jj < kBatch; ++jj) {
+              p0[jj] = *(const uint4*)(qh[jj] + 8 * c0);
+              p1[jj] = *(const uint4*)(qh[jj] + 8 * c1);
+            }
+          }
+#pragma unroll
+          for (int jj = 0; jj < kBatch; ++jj) {
+            const int Rl = rl0 + (it0 + jj) * kRowStep;
+            if (!live[it0 + jj]) p0[jj] = p1[jj] = make_uint4(0, 0, 0, 0);
+            q_stage[Rl * kChunks + (c0 ^ wide_swz<kD>(Rl))] = va_u32x4{p0[jj].x, p0[jj].y, p0[jj].z, p0[jj].w};
+            q_stage[Rl * kChunks + (c1 ^ wide_swz<kD>(Rl))] = va_u32x4{p1[jj].x, p1[jj].y, p1[jj].z, p1[jj].w};
+          }
+        }
+      } else {
+        // mRoPE computes its cosines and sines (no table to wait for): row by row
+        for (int idx = tid; idx < 128 * (kChunks / 2); idx += kWideThreads) {  // two pieces per step
+          const int Rl = idx / (kChunks / 2), x = idx - Rl * (kChunks / 2);
+          const int R = kWaveRows * (Rl / 32) + 32 * pass + Rl % 32;  // block `pass` of every wave
+          const int iq = R / G, g = R - iq * G;
+          int c0 = 2 * x, c1 = 2 * x + 1;
+          uint4 p0 = make_uint4(0, 0, 0, 0), p1 = p0;
+          if (iq < n_q) {
+            const int subrow = (lflags & VA_LINK_INDIRECT) ? a.qrefs[qref + iq] : qref + iq;
+            const long long src_row = a.sub_worker[subrow];
+            const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
+            const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
+            rotated_query_unit<E>(a.rope, qh, x, p, c0, c1, p0, p1);
+          }
+          q_stage[Rl * kChunks + (c0 ^ wide_swz<kD>(Rl))] = va_u32x4{p0.x, p0.y, p0.z, p0.w};
+          q_stage[Rl * kChunks + (c1 ^ wide_swz<kD>(Rl))] = va_u32x4{p1.x, p1.y, p1.z, p1.w};
+        }
       }
       ring_barrier<kAnyInFlight>();
       {
