@@ -244,7 +244,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         // -> query pieces and cos|sin entries) is paid once per batch, not once per row (row by row
         // this set-up was an eighth of the kernel on long views of many blocks).
         constexpr int kUnits = kChunks / 2, kRowStep = kWideThreads / kUnits, kIts = 128 / kRowStep;
-        constexpr int kBatch = kIts < 4 ? kIts : 4;
+        constexpr int kBatch = kIts < 2 ? kIts : 2;
         static_assert(kWideThreads % kUnits == 0 && 128 % kRowStep == 0 && kIts % kBatch == 0, "staging pattern");
         const int x = tid % kUnits, rl0 = tid / kUnits;
         const int pair_units = a.rope.rotary_dim / 16;
@@ -364,7 +364,11 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       row_ahead = row_of(k + 1 + kWideAhead);
       // only the loads of the tiles requested after tile k (up to kWideAhead - 1 of them) may still be outstanding
       if (k + kWideAhead - 1 < n_tiles) {
+#if VA_WIDE_EXPERIMENT == 6
+        ring_barrier<(kWideAhead - 1) * kL / 2>();
+#else
         ring_barrier<(kWideAhead - 1) * kL>();
+#endif
       } else if (kWideAhead > 2 && k + 1 < n_tiles) {
         ring_barrier<kL>();
       } else {
@@ -383,11 +387,23 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       const long long row = row_ahead;
       const int t = tok_begin + (k + 1 + kWideAhead) * kWideTokens + 16 * wave_half;
       const int page = ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + (t >> p_shift)];
+#if VA_WIDE_EXPERIMENT == 6
+      const int zero = ring_barrier_zero<(kWideAhead - 1) * kL / 2>();
+#else
       const int zero = ring_barrier_zero<(kWideAhead - 1) * kL>();
+#endif
       const uint32_t dst = wave_lds + ((k + kWideAhead) % kWideBuffers) * Sh::kBufferBytes;
       const char* base = wave_pool + row * row_bytes;
+#if VA_WIDE_EXPERIMENT == 6  // half of the loads (timing only)
+#pragma unroll
+      for (int u = 0; u < kL; u += 2) load_to_lds(base, ld_off[u], dst + u * 1024);
+#elif VA_WIDE_EXPERIMENT == 7  // all loads, to one LDS address and from one row (timing only)
+#pragma unroll
+      for (int u = 0; u < kL; ++u) load_to_lds(base, ld_off[0], dst);
+#elif VA_WIDE_EXPERIMENT != 5
 #pragma unroll
       for (int u = 0; u < kL; ++u) load_to_lds(base, ld_off[u], dst + u * 1024);
+#endif
       row_ahead = ((long long)(page + zero) << p_shift) + (t & (P - 1));
     };
     // iterations [1, i_steady_end) may take it: tiles i + 1 + kWideAhead and i + 2 + kWideAhead are plain,
@@ -507,9 +523,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         auto exp_piece = [&](int r) __attribute__((always_inline)) {
 #pragma unroll
           for (int b = 0; b < kB; ++b) {
-            // sc holds s - m_ref already; issued from assembly so that it stays where it is written,
-            // between two score products
-            asm volatile("v_exp_f32 %0, %0" : "+v"(sc[b][r]));
+            sc[b][r] = __builtin_amdgcn_exp2f(sc[b][r]);  // sc holds s - m_ref already
             if (r > 0) sum[b] += sc[b][r - 1];
             if (r >= 2 && r % 2 == 0) pw[b][r / 2 - 1] = Mma<E>::pack(sc[b][r - 2], sc[b][r - 1]);
           }
@@ -519,14 +533,19 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         // the following ring buffer holds and are never looked at (sixteen idle products per link
         // against a second copy of this phase and the register moves where the two would meet).
         read_k(i + 1);
-#pragma unroll
-        for (int idx = 0; idx < kVAhead; ++idx) read_vfrag(idx);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           if (r % kPiecesPerStep == 0) score_step(r / kPiecesPerStep);
           __builtin_amdgcn_sched_barrier(0);
           exp_piece(r);
+          // the first V fragments are requested once half of the K fragments have been consumed: the
+          // counter of outstanding LDS reads holds fifteen, and a wait for the first K fragment
+          // with more than that in flight becomes a wait for the excess as well
+          if (r == 8) {
+#pragma unroll
+            for (int idx = 0; idx < kVAhead; ++idx) read_vfrag(idx);
+          }
           __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
