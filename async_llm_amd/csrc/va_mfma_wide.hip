@@ -67,6 +67,10 @@ __device__ __forceinline__ int wide_swz(int r) {
   return (r >> 1) & 7;
 }
 
+// Ring buffer of a tile (tile numbers are never negative: the unsigned remainder is one instruction
+// for a power-of-two ring, the signed one five).
+__device__ __forceinline__ uint32_t ring_slot(int tile) { return (uint32_t)tile % (uint32_t)kWideBuffers; }
+
 // V tiles are read with transposing loads (16 lanes fetch 4 tokens x 16 dims, 32 bytes per token):
 // moving token r's pieces by 2 (r % 4) puts the four rows of such a fetch side by side in one
 // 128-byte window.
@@ -210,7 +214,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       return uniform_pages && tok_begin + (i + 1) * kWideTokens - 1 <= t_last;
     };
     auto issue = [&](int i, long long row) __attribute__((always_inline)) {
-      const uint32_t dst = wave_lds + (i % kWideBuffers) * Sh::kBufferBytes;
+      const uint32_t dst = wave_lds + ring_slot(i) * Sh::kBufferBytes;
       if (tile_is_plain(i)) {
         const char* base = wave_pool + row * row_bytes;
 #pragma unroll
@@ -392,7 +396,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
 #else
       const int zero = ring_barrier_zero<(kWideAhead - 1) * kL>();
 #endif
-      const uint32_t dst = wave_lds + ((k + kWideAhead) % kWideBuffers) * Sh::kBufferBytes;
+      const uint32_t dst = wave_lds + ring_slot(k + kWideAhead) * Sh::kBufferBytes;
       const char* base = wave_pool + row * row_bytes;
 #if VA_WIDE_EXPERIMENT == 6  // half of the loads (timing only)
 #pragma unroll
@@ -419,7 +423,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     va_f32x16 sc_next[kB];  // scores of the next tile, accumulating
     va_u32x4 kf[kSteps];
     auto read_k = [&](int tile) __attribute__((always_inline)) {
-      const char* kt = lds + (tile % kWideBuffers) * Sh::kBufferBytes;
+      const char* kt = lds + ring_slot(tile) * Sh::kBufferBytes;
 #pragma unroll
       for (int s = 0; s < kSteps; ++s) kf[s] = *(const va_u32x4*)(kt + k_row_byte + 16 * ((2 * s + h) ^ swz_j));
     };
@@ -501,7 +505,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         resume = false;
 
         // V^T fragments of this tile, kVAhead of them in flight: fragment idx = (step kk, dim tile t)
-        const uint32_t vt = lds_base + (i % kWideBuffers) * Sh::kBufferBytes + Sh::kTileBytes;
+        const uint32_t vt = lds_base + ring_slot(i) * Sh::kBufferBytes + Sh::kTileBytes;
         const uint32_t vt_even = vt + v_even, vt_odd = vt + v_odd;
         constexpr int kFrags = 2 * kDimTiles;
         constexpr int kMaxFirst = kFrags > 2 ? 2 : kFrags - 1;  // first product the early maxima follow
