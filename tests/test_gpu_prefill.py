@@ -171,3 +171,43 @@ def test_prefill_head_layouts(dtype, heads, rotary):
         specs = make_specs(common, lengths, turn, page, False)
         *_, meta = run_prefill_parity(op, cpu_pool, dev_pool, specs, 1e4, gen, scale=1.0)
         assert meta.launch.counts.kernel == 2 and meta.launch.counts.n_wide_items > 0
+
+
+@pytest.mark.parametrize("dtype,heads,rotary,mrope", [
+    (torch.bfloat16, (8, 2, 256), 256, False),
+    (torch.float16, (8, 4, 128), 64, False),
+    (torch.bfloat16, (4, 2, 64), 64, False),
+    (torch.bfloat16, (8, 2, 256), 128, True),
+])
+def test_long_links_of_whole_pages(dtype, heads, rotary, mrope):
+    """Context blocks of hundreds of tokens on 16-token pages: the wide kernel walks
+    the interior tiles of such a link with its branch-free ring step (page lookup
+    a step ahead, uniform loads), the first, masked and last tiles with the
+    general one.  Unit-variance data makes the per-row reference maxima rise
+    inside those runs too (rescale and resume in the middle of a link)."""
+    page = 16
+    op, cpu_pool, dev_pool, gen = make_op_and_pool(
+        DEV, dtype, heads, page, 200, 1e4, rotary_dim=rotary, mrope_section=(32, 16, 16) if mrope else None,
+        seed=4242, scale=1.0 if heads[2] <= 64 else 0.5, max_pos=4096)
+    blocks, first = [], 0
+    for length in (701, 333, 96):
+        b = CacheBlock(DEV, page)
+        n_pages = -(-length // page)
+        b.grow_pages(torch.arange(first, first + n_pages) * page, length)
+        if mrope:
+            b.mrope_span_override = length // 3 + 5
+        blocks.append(b)
+        first += n_pages
+    specs = []
+    for worker, (length, prefix) in enumerate(((96, 200), (17, 330))):
+        n_pages = -(-(prefix + length) // page)
+        pages = torch.arange(first, first + n_pages, dtype=torch.int32) * page
+        first += n_pages
+        rel = None
+        if mrope and worker == 0:
+            p = torch.arange(length)
+            rel = torch.stack([p // 8, p // 4, p % 4])
+        specs.append(PrefillSpec(blocks[worker:], pages, length, prefix, prefix // 2 if mrope else prefix, rel))
+    assert first <= 200
+    *_, meta = run_prefill_parity(op, cpu_pool, dev_pool, specs, 1e4, gen, scale=1.0 if heads[2] <= 64 else 0.5)
+    assert meta.launch.counts.kernel == 2 and meta.launch.counts.n_wide_items > 0
