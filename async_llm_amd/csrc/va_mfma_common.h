@@ -28,26 +28,23 @@ struct Mma<BF16> {
   // Same product with the accumulator pinned in the accumulation registers (AGPRs).  Written as
   // assembly because the register allocator otherwise treats AGPRs as spill space for a long-lived
   // accumulator and copies all of it to VGPRs and back around every tile.  The compiler cannot
-  // insert wait states for code it does not see: the leading s_nop covers the two wait states
-  // between a vector-ALU write of an operand (the transposed V fragment, the packed P) and the
-  // matrix pipe reading it, and callers wait (accumulator_fence) before reading the accumulator
-  // with anything but another product.
+  // insert wait states for an instruction it does not see: the matrix pipe must not read an operand
+  // in the two wait states after a vector-ALU instruction wrote it, and ANY product can be preceded
+  // by such a write -- the transposed V fragment, the packed P, but also a register copy the
+  // allocator places in front of the statement (an operand parked in an AGPR is brought back with
+  // v_accvgpr_read right there).  Every product issued from assembly therefore carries its own
+  // `s_nop 1`; without it results depended on the register allocation of the build.  Callers wait
+  // (accumulator_fence) before reading an accumulator with anything but another product.
   static __device__ __forceinline__ void run32_acc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
-  // ... without the wait states: for products whose operands no vector-ALU instruction has written
-  // since an earlier product of the same run was issued
-  static __device__ __forceinline__ void run32_acc_next(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-  }
   // The same with the accumulator in ordinary vector registers (for results the vector ALU reads
-  // next, the scores); `first`: the sum starts from zero.  No leading s_nop: the operands of these
-  // products come from LDS reads and from registers written long before.
+  // next, the scores); `first`: the sum starts from zero.
   static __device__ __forceinline__ void run32_vacc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ void run32_vacc_first(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
   }
   template <typename A, typename B>
   static __device__ __forceinline__ va_f32x4 run(const A& a, const B& b, va_f32x4 c) {
@@ -76,14 +73,11 @@ struct Mma<F16> {
   static __device__ __forceinline__ void run32_acc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
-  static __device__ __forceinline__ void run32_acc_next(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-  }
   static __device__ __forceinline__ void run32_vacc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ void run32_vacc_first(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
   }
   template <typename A, typename B>
   static __device__ __forceinline__ va_f32x4 run(const A& a, const B& b, va_f32x4 c) {

@@ -572,12 +572,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
           const int kk = idx / kDimTiles, t = idx % kDimTiles;
 #pragma unroll
           for (int b = 0; b < kB; ++b) {
-            // P was packed by the vector ALU just before the first product; V fragments come from LDS
-            if (idx == 0) {
-              Mma<E>::run32_acc(vfr[idx % kVAhead], pf[kk][b], o[b][t]);
-            } else {
-              Mma<E>::run32_acc_next(vfr[idx % kVAhead], pf[kk][b], o[b][t]);
-            }
+            Mma<E>::run32_acc(vfr[idx % kVAhead], pf[kk][b], o[b][t]);
           }
           __builtin_amdgcn_sched_barrier(0);
           if (idx + kVAhead < kFrags) read_vfrag(idx + kVAhead);
