@@ -254,6 +254,34 @@ __device__ __forceinline__ void load_to_lds(const void* base, uint32_t lane_offs
                "s"(lds_base)
                : "memory");
 }
+// Up to four such loads behind ONE setting of M0: the instruction's immediate offset is added to
+// the pool address AND to the LDS address, so load u of a group lands 1024 u bytes further on when
+// its per-lane offset has had 1024 u taken off beforehand (grouped_lane_offset).  Two scalar
+// instructions per group instead of three per load.
+__device__ __forceinline__ uint32_t grouped_lane_offset(uint32_t lane_offset, int u) { return lane_offset - 1024u * (u % 4); }
+template <int kCount>
+__device__ __forceinline__ void load_group_to_lds(const void* base, const uint32_t* adjusted_offsets, uint32_t lds_base) {
+  static_assert(kCount == 1 || kCount == 2 || kCount == 4, "loads per group");
+  if constexpr (kCount == 4) {
+    asm volatile(
+        "s_mov_b32 m0, %5\n\ts_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, %4\n\t"
+        "global_load_lds_dwordx4 %1, %4 offset:1024\n\t"
+        "global_load_lds_dwordx4 %2, %4 offset:2048\n\t"
+        "global_load_lds_dwordx4 %3, %4 offset:3072" ::"v"(adjusted_offsets[0]),
+        "v"(adjusted_offsets[1]), "v"(adjusted_offsets[2]), "v"(adjusted_offsets[3]), "s"(base), "s"(lds_base)
+        : "memory");
+  } else if constexpr (kCount == 2) {
+    asm volatile(
+        "s_mov_b32 m0, %3\n\ts_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, %2\n\t"
+        "global_load_lds_dwordx4 %1, %2 offset:1024" ::"v"(adjusted_offsets[0]),
+        "v"(adjusted_offsets[1]), "s"(base), "s"(lds_base)
+        : "memory");
+  } else {
+    load_to_lds(base, adjusted_offsets[0], lds_base);
+  }
+}
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }

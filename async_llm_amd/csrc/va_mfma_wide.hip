@@ -138,7 +138,16 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   uint32_t ld_off[kL];
 #pragma unroll
   for (int u = 0; u < kL; ++u)
-    ld_off[u] = (uint32_t)((u * Sh::kRowsPerLoad + ld_row0) * row_bytes + 16 * (ld_x0 ^ ld_swz(u * Sh::kRowsPerLoad)));
+    ld_off[u] = grouped_lane_offset(
+        (uint32_t)((u * Sh::kRowsPerLoad + ld_row0) * row_bytes + 16 * (ld_x0 ^ ld_swz(u * Sh::kRowsPerLoad))), u);
+  // the loads of a plain tile go out in groups of up to four behind one setting of M0; a group's
+  // rows start at least 1024 bytes apart in the pool (kRowsPerLoad rows of at least 2 D bytes), so
+  // the offsets stay non-negative after the adjustment
+  constexpr int kLoadGroup = kL >= 4 ? 4 : kL;
+  auto issue_plain = [&](const char* base, uint32_t dst) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < kL; u += kLoadGroup) load_group_to_lds<kLoadGroup>(base, ld_off + u, dst + u * 1024);
+  };
   // LDS offsets of what this lane reads from a tile
   const int swz_j = wide_swz<kD>(j);
   const int k_row_byte = j * kRowBytes;
@@ -217,8 +226,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       const uint32_t dst = wave_lds + ring_slot(i) * Sh::kBufferBytes;
       if (tile_is_plain(i)) {
         const char* base = wave_pool + row * row_bytes;
-#pragma unroll
-        for (int u = 0; u < kL; ++u) load_to_lds(base, ld_off[u], dst + u * 1024);
+        issue_plain(base, dst);
       } else {
         const int t0 = tok_begin + i * kWideTokens + 16 * wave_half;
 #pragma unroll
@@ -368,11 +376,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       row_ahead = row_of(k + 1 + kWideAhead);
       // only the loads of the tiles requested after tile k (up to kWideAhead - 1 of them) may still be outstanding
       if (k + kWideAhead - 1 < n_tiles) {
-#if VA_WIDE_EXPERIMENT == 6
-        ring_barrier<(kWideAhead - 1) * kL / 2>();
-#else
         ring_barrier<(kWideAhead - 1) * kL>();
-#endif
       } else if (kWideAhead > 2 && k + 1 < n_tiles) {
         ring_barrier<kL>();
       } else {
@@ -391,22 +395,11 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       const long long row = row_ahead;
       const int t = tok_begin + (k + 1 + kWideAhead) * kWideTokens + 16 * wave_half;
       const int page = ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + (t >> p_shift)];
-#if VA_WIDE_EXPERIMENT == 6
-      const int zero = ring_barrier_zero<(kWideAhead - 1) * kL / 2>();
-#else
       const int zero = ring_barrier_zero<(kWideAhead - 1) * kL>();
-#endif
       const uint32_t dst = wave_lds + ring_slot(k + kWideAhead) * Sh::kBufferBytes;
       const char* base = wave_pool + row * row_bytes;
-#if VA_WIDE_EXPERIMENT == 6  // half of the loads (timing only)
-#pragma unroll
-      for (int u = 0; u < kL; u += 2) load_to_lds(base, ld_off[u], dst + u * 1024);
-#elif VA_WIDE_EXPERIMENT == 7  // all loads, to one LDS address and from one row (timing only)
-#pragma unroll
-      for (int u = 0; u < kL; ++u) load_to_lds(base, ld_off[0], dst);
-#elif VA_WIDE_EXPERIMENT != 5
-#pragma unroll
-      for (int u = 0; u < kL; ++u) load_to_lds(base, ld_off[u], dst + u * 1024);
+#if VA_WIDE_EXPERIMENT != 5
+      issue_plain(base, dst);
 #endif
       row_ahead = ((long long)(page + zero) << p_shift) + (t & (P - 1));
     };
