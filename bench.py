@@ -46,8 +46,8 @@ MEASURED_TRAFFIC_BYTES = {
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=40)
-    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default: about a second of GPU time)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default: steps / 10)")
     ap.add_argument("--workload", default="batched_decode",
                     choices=["batched_decode", "mrope_decode", "view_prefill", "plumbing_decode", "mixed_batch",
                              "copy_calibration", "block_merge"])
@@ -292,12 +292,32 @@ def main() -> int:
         return 2
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload in ("copy_calibration", "block_merge"):
+        args.steps = 40 if args.steps is None else args.steps
+        args.warmup = 8 if args.warmup is None else args.warmup
     if args.workload == "copy_calibration":
         return copy_calibration(dev, args.steps)
     if args.workload == "block_merge":
         return block_merge(dev, args.steps, args.warmup, args.layers, not args.no_cpu_baseline)
     wl = build_workload(args.workload, dev, args.layers, args.kernel)
     layers = args.layers
+
+    # The shader clock idles at ~0.15 GHz and takes some milliseconds of load to reach its working
+    # frequency: run the step untimed for a while first (not counted in W or K), so that a short
+    # K measures the kernels and not the ramp.
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < 0.2:
+        for i in range(8):
+            wl.forward(i % layers)
+        torch.cuda.synchronize()
+    if args.steps is None:  # about a second of steps
+        t0 = time.perf_counter()
+        for i in range(8):
+            wl.forward(i % layers)
+        torch.cuda.synchronize()
+        args.steps = max(20, min(2000, int(8 / (time.perf_counter() - t0))))
+    if args.warmup is None:
+        args.warmup = max(4, args.steps // 10)
 
     # whole step (store + attention + merge), wall clock around K steps
     for i in range(args.warmup):
