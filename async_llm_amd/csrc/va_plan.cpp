@@ -310,16 +310,21 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
         for (int32_t t0 = 0; t0 < len; t0 += per_w) emit_range(ti, t0, std::min(len, t0 + per_w));
   }
 
-  // chains are split only when tiles alone cannot fill the machine
-  int32_t chain_split = 1;
+  // Chains are split only when their tiles alone cannot fill the machine, and then by tokens: a
+  // tile gets one piece per `chain_budget` tokens it walks, so the tiles of a short request stay
+  // whole while those of a long one are cut (in a mixed batch the views differ by a factor of
+  // thirty; a uniform cut leaves the launch waiting for the longest).  The number of extra pieces
+  // over all tiles is at most chain_tokens / chain_budget <= want <= target.
+  int64_t chain_budget = INT64_MAX;
   if (chain_tiles > 0) {
-    const int64_t want = std::max<int64_t>(1, target - (int64_t)out.items.size());
-    if (chain_tiles < want) {
-      const int64_t avg = chain_tokens / chain_tiles;
-      chain_split = (int32_t)std::min<int64_t>((want + chain_tiles - 1) / chain_tiles,
-                                               std::max<int64_t>(1, avg / (8 * gran)));
-    }
+    // three rounds of work items over the CUs a head leaves to a launch of one workgroup per CU
+    const int64_t rounds = 3 * std::max(1, 256 / shape->num_kv_heads);
+    const int64_t want = std::max<int64_t>(1, std::min<int64_t>(target - (int64_t)out.items.size(), rounds));
+    if (chain_tiles < want) chain_budget = std::max<int64_t>((chain_tokens + want - 1) / want, 4 * gran);
   }
+  // cuts inside a segment keep to multiples of 16 tokens where the kernels profit (pages of 16
+  // tokens or more: a piece that starts on such a boundary is fetched with uniform loads)
+  const bool align_cuts = shape->page_size >= 16 && (shape->page_size & (shape->page_size - 1)) == 0;
   for (auto& ch : chains) {
     const int32_t nq = s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]];
     cut_tiles(nq, tiles);
@@ -340,17 +345,30 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
       std::vector<int32_t> rows;
       for (int32_t r = a; r < b; ++r) rows.push_back((int32_t)s->sub_worker[s->qo_indptr[ch[0]] + r]);
       if (all.empty()) continue;
-      const int32_t parts = (int32_t)std::max<int64_t>(1, std::min<int64_t>(chain_split, tile_tokens / (4 * gran)));
+      const int32_t parts = (int32_t)std::max<int64_t>(
+          1, std::min<int64_t>((tile_tokens + chain_budget / 2) / chain_budget, tile_tokens / (4 * gran)));
       if (parts == 1) {
         emit(b - a, all, std::move(rows));
         continue;
       }
-      const int32_t per = round_up((tile_tokens + parts - 1) / parts, gran);
+      // an aligned cut may leave up to 15 tokens of a piece's room unused: the room allows for it, so
+      // that a tile never ends up in more than `parts` pieces
+      const int32_t per = round_up((tile_tokens + parts - 1) / parts + (align_cuts ? 15 : 0), gran);
       std::vector<Link> cur;
       int32_t room = per;
       for (auto l : all) {
+        const bool aligned = align_cuts && !(l.flags & VA_LINK_SLOTS);
         while (l.tok_begin < l.tok_end) {
-          const int32_t take = std::min(room, l.tok_end - l.tok_begin);
+          int32_t take = std::min(room, l.tok_end - l.tok_begin);
+          if (aligned && take < l.tok_end - l.tok_begin) {
+            take = take / 16 * 16;  // l.tok_begin is a multiple of 16: segments start at 0, cuts keep it so
+            if (take == 0) {        // under 16 tokens of room left: the piece ends here
+              emit(b - a, cur, std::vector<int32_t>(rows));
+              cur.clear();
+              room = per;
+              continue;
+            }
+          }
           Link piece = l;
           piece.tok_end = l.tok_begin + take;
           cur.push_back(piece);
@@ -662,8 +680,9 @@ extern "C" int64_t va_plan_fixed_words(const VaPlanCapacity* cap) {
 //     chunk >= total_tokens / target, plus one for the halved last chunk, so items <= 2 tiles + target
 //     with tiles <= sub-requests; every item carries one link; a query row enters the partial list
 //     once per chunk of its run;
-//   * chains: tiles of up to wide_tile rows (the last one of a chain may be narrow), each split
-//     into at most ceil(target / tiles) pieces, so items <= tiles + target per class; a tile has
+//   * chains: tiles of up to wide_tile rows (the last one of a chain may be narrow); a tile is
+//     split into round(its tokens / budget) pieces with budget >= all chain tokens / target, so
+//     the extra pieces number at most target and items <= tiles + target per class; a tile has
 //     one link per member plus one per cut; a split tile's rows enter the partial list once per piece.
 extern "C" int va_plan_capacity(const VaShape* shape, const VaPlanParams* params, const VaPlanLimits* lim,
                                 VaPlanCapacity* capacity) {

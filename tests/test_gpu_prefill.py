@@ -125,16 +125,19 @@ def test_mixed_batch_single_launch(kernel):
     assert_close(lse[W:], el_p, op.dtype, "prefill lse")
 
 
+@pytest.mark.parametrize("page", [16, 4])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_split_chains_with_unaligned_pieces(dtype):
+def test_split_chains(dtype, page):
     """Few query tiles over long context: the planner cuts each tile's chain of
-    segments into several work items.  Segment lengths that are no multiples of
-    16 make later pieces start inside a 16-token page group, which the kernels
-    must address token by token."""
+    segments into several work items.  With pages of 16 tokens its cuts stay on
+    16-token boundaries inside a segment (such pieces are fetched with uniform
+    loads); with smaller pages they fall where the token budget ends, segment
+    lengths that are no multiples of 16 make later pieces start anywhere, and
+    the kernels address them token by token."""
     from tests.test_native_abi_cpu import decode_plan
 
-    page, heads = 16, (8, 2, 128)
-    op, cpu_pool, dev_pool, gen = make_op_and_pool(DEV, dtype, heads, page, 320, 1e6, seed=77, kernel="auto",
+    heads = (8, 2, 128)
+    op, cpu_pool, dev_pool, gen = make_op_and_pool(DEV, dtype, heads, page, 5200 // page, 1e6, seed=77, kernel="auto",
                                                    max_pos=8192)
     lengths = (1999, 1501, 777)
     context, first = [], 0
@@ -145,13 +148,17 @@ def test_split_chains_with_unaligned_pieces(dtype):
         first += n_pages
         context.append(b)
     for new_tokens in (24, 3):  # a wide tile, then a narrow one
-        pages = torch.arange(first, first + 4, dtype=torch.int32) * page
+        pages = torch.arange(first, first + 64 // page, dtype=torch.int32) * page
         specs = [PrefillSpec(context, pages, new_tokens, 21)]
         *_, meta = run_prefill_parity(op, cpu_pool, dev_pool, specs, 1e6, gen)
         h, items, links, *_ = decode_plan(meta.launch.blob.cpu().numpy())
         real = [it for it in items if it[2] > 0]
         assert len(real) > 1, "the chain was not split"
-        assert any(l[1] % 16 for it in real for l in links[it[0]: it[0] + it[1]]), "no unaligned piece in this plan"
+        starts = [l[1] for it in real for l in links[it[0]: it[0] + it[1]]]
+        if page >= 16:
+            assert all(t % 16 == 0 for t in starts), "a cut left its 16-token boundary"
+        else:
+            assert any(t % 16 for t in starts), "no unaligned piece in this plan"
 
 
 @pytest.mark.parametrize("dtype,heads,rotary", [
