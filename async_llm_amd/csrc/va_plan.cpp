@@ -320,7 +320,8 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     // three rounds of work items over the CUs a head leaves to a launch of one workgroup per CU
     const int64_t rounds = 3 * std::max(1, 256 / shape->num_kv_heads);
     const int64_t want = std::max<int64_t>(1, std::min<int64_t>(target - (int64_t)out.items.size(), rounds));
-    if (chain_tiles < want) chain_budget = std::max<int64_t>((chain_tokens + want - 1) / want, 4 * gran);
+    // (a piece pays its own set-up -- the query tile is staged again -- so none is made for under ~1000 tokens)
+    if (chain_tiles < want) chain_budget = std::max<int64_t>((chain_tokens + want - 1) / want, 16 * gran);
   }
   // cuts inside a segment keep to multiples of 16 tokens where the kernels profit (pages of 16
   // tokens or more: a piece that starts on such a boundary is fetched with uniform loads)

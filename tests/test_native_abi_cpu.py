@@ -309,3 +309,46 @@ def test_compute_entry_points_refuse_cpu_tensors():
 
     with pytest.raises(native.ViewAttnError, match="GPU only"):
         apply_rope_correction(torch.zeros(2, 1, 8), torch.zeros(2, dtype=torch.int64), torch.zeros(4, 8))
+
+
+def test_prefill_tiles_are_cut_by_tokens_on_page_group_boundaries():
+    """Two prefill requests of one 32-row tile each, one over 30000 context tokens
+    in three segments of odd lengths, one over 700: too few tiles to fill the
+    machine, so the planner splits them by tokens.  The long tile must come out
+    in many pieces of similar weight, the short one whole; with pages of 16
+    tokens every cut inside a segment lies on a 16-token boundary, with pages of
+    4 it need not; every visible pair is covered once either way."""
+    for page in (16, 4):
+        qo, kvp, kvi, lens, flags, chain, sw = [0], [0], [], [], [], [], []
+        n_rows = 0
+        for r, segments in enumerate(((11111, 9999, 8890), (700,))):
+            rows = list(range(n_rows, n_rows + 8))
+            n_rows += 8
+            for L in segments:
+                kvi += list(range(len(kvi), len(kvi) + -(-L // page)))
+                kvp.append(len(kvi)); lens.append(L); flags.append(0); chain.append(r)
+                sw += rows; qo.append(len(sw))
+            kvi += list(range(len(kvi), len(kvi) + -(-(40 + 8) // page)))
+            kvp.append(len(kvi)); lens.append(48); flags.append(1); chain.append(r)
+            sw += rows; qo.append(len(sw))
+        rc, blob, counts = build_plan(qo, kvp, kvi, lens, flags, chain, sw, n_rows, heads=(16, 4, 256), page=page,
+                                      dtype=native.VA_BF16, kernel=native.VA_KERNEL_MFMA)
+        assert rc == 0
+        check_coverage(blob, qo, kvp, lens, flags, sw, n_rows)
+        h, items, links, *_ = decode_plan(blob)
+        real = [it for it in items if it[2] > 0]
+        weight = {}
+        for it in real:
+            ls = links[it[0]: it[0] + it[1]]
+            tokens = sum(int(l[2] - l[1]) for l in ls)
+            long_one = any(int(l[0]) < kvp[3] for l in ls)  # kv_begin inside the first request's tables
+            weight.setdefault(long_one, []).append(tokens)
+        assert len(weight[False]) == 1, "the short tile was cut"
+        assert len(weight[True]) >= 20, "the long tile was not cut by its tokens"
+        assert max(weight[True]) <= 1.3 * min(w for w in weight[True][:-1]), weight[True]
+        inner = [int(l[1]) for it in real for l in links[it[0]: it[0] + it[1]] if l[1] > 0]
+        assert inner, "no cut inside a segment"
+        if page >= 16:
+            assert all(t % 16 == 0 for t in inner)
+        else:
+            assert any(t % 16 for t in inner)
