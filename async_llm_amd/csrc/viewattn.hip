@@ -324,14 +324,15 @@ __global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// merge of partial states: one workgroup of four waves per (row, q head)
+// merge of partial states: one workgroup of kMergeWaves waves per (row, q head)
 // ---------------------------------------------------------------------------
 // The launch is short and made of dependent loads (row list -> partial states), so it is laid out
-// for latency: wave w folds partials w, w + 4, ... of the row, eight per round with all their loads
-// in flight together, and the four running states meet in LDS.  Lane l owns dims l, l + 64, ...
-constexpr int kMergeWaves = 4;
-
-template <typename E>
+// for latency: wave w folds partials w, w + kMergeWaves, ... of the row, eight per round with all
+// their loads in flight together, and the running states meet in LDS.  Lane l owns dims l, l + 64, ...
+// Four waves for a decode batch (few rows, up to dozens of partial states each); one wave when the
+// rows are many (split prefill tiles: thousands of rows of a few states each), where four times as
+// many rows in flight per CU count for more than the parallel fold.
+template <typename E, int kMergeWaves>
 __global__ __launch_bounds__(64 * kMergeWaves) void merge_kernel(MergeArgs a) {
   using S = typename E::storage;
   const long long row = blockIdx.x;
@@ -374,28 +375,30 @@ __global__ __launch_bounds__(64 * kMergeWaves) void merge_kernel(MergeArgs a) {
       mm = m_new;
     }
   }
-  // fold the waves' states: wave 0 collects
-  __shared__ float s_ml[kMergeWaves][2];
-  __shared__ float s_av[kMergeWaves][4][64];
-  if (wave > 0) {
-    if (lane == 0) {
-      s_ml[wave][0] = mm;
-      s_ml[wave][1] = ll;
+  if constexpr (kMergeWaves > 1) {
+    // fold the waves' states: wave 0 collects
+    __shared__ float s_ml[kMergeWaves][2];
+    __shared__ float s_av[kMergeWaves][4][64];
+    if (wave > 0) {
+      if (lane == 0) {
+        s_ml[wave][0] = mm;
+        s_ml[wave][1] = ll;
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) s_av[wave][k][lane] = av[k];
     }
+    __syncthreads();
+    if (wave > 0) return;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) s_av[wave][k][lane] = av[k];
-  }
-  __syncthreads();
-  if (wave > 0) return;
+    for (int w = 1; w < kMergeWaves; ++w) {
+      const float mw = s_ml[w][0], lw = s_ml[w][1];
+      const float m_new = fmaxf(mm, mw);
+      const float sa = exp2f(mm - m_new), sb = exp2f(mw - m_new);
+      ll = ll * sa + lw * sb;
 #pragma unroll
-  for (int w = 1; w < kMergeWaves; ++w) {
-    const float mw = s_ml[w][0], lw = s_ml[w][1];
-    const float m_new = fmaxf(mm, mw);
-    const float sa = exp2f(mm - m_new), sb = exp2f(mw - m_new);
-    ll = ll * sa + lw * sb;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) av[k] = av[k] * sa + s_av[w][k][lane] * sb;
-    mm = m_new;
+      for (int k = 0; k < 4; ++k) av[k] = av[k] * sa + s_av[w][k][lane] * sb;
+      mm = m_new;
+    }
   }
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
@@ -434,7 +437,12 @@ int launch_generic(const AttnArgs& a, int n_items, hipStream_t stream) {
 
 template <typename E>
 int launch_merge(const MergeArgs& a, int n_rows, hipStream_t stream) {
-  hipLaunchKernelGGL(merge_kernel<E>, dim3((unsigned)n_rows, (unsigned)a.num_q_heads), dim3(64 * kMergeWaves), 0, stream, a);
+  const dim3 grid((unsigned)n_rows, (unsigned)a.num_q_heads);
+  if ((int64_t)n_rows * a.num_q_heads >= 8192) {
+    hipLaunchKernelGGL((merge_kernel<E, 1>), grid, dim3(64), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((merge_kernel<E, 4>), grid, dim3(256), 0, stream, a);
+  }
   return check_hip(hipGetLastError(), "merge launch");
 }
 
