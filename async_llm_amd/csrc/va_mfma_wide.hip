@@ -1,28 +1,28 @@
 // Wide matrix-core view attention: query tiles of 128 (head_dim 256) or 256 MFMA rows, for
 // view-conditioned prefill (rows / G new tokens x G heads per workgroup).
 //
-// One workgroup of four waves per (work item, kv head); wave w owns one or two blocks of 32
-// MFMA rows (row R = tile row R / G, head R % G).  All waves walk the same 32-token
-// K/V tiles, which travel pool -> LDS directly (global_load_lds_dwordx4) into a ring of four
-// buffers: three tiles are in flight while one is computed, one barrier per tile.
+// One workgroup of four waves per (work item, kv head), one wave per SIMD; wave w owns one
+// (head_dim 256) or two blocks of 32 MFMA rows (row R = tile row R / G, head R % G).  All waves walk
+// the same 32-token K/V tiles, which travel pool -> LDS directly (global_load_lds_dwordx4) into a
+// ring of four buffers: two tiles are in flight while the scores of a third and the products of a
+// fourth are computed, one barrier per tile.
 //
 //   S^T[32 tokens, 32 rows] = K . Q^T    v_mfma_f32_32x32x16, K from LDS as the A operand; each K
 //                                        fragment is read once and used for all row blocks, whose
 //                                        rotated queries are pinned in registers as B operands
-//   online softmax per row (row = lane % 32; the other half-wave holds the other 16 tokens)
+//   softmax per row against a reference maximum that is raised only when a tile exceeds it by far
+//   (row = lane % 32; the other half-wave holds the other 16 tokens)
 //   O^T[D, 32 rows] += V^T . P^T         2 token steps x D/32 dim tiles; P is already laid out as
-//                                        the B operand; V rows are read from LDS as 8 tokens x D/32
-//                                        dims per lane, transposed in registers with v_perm_b32, and
-//                                        each transposed fragment again serves all row blocks
+//                                        the B operand; V^T fragments come from transposing LDS
+//                                        reads (ds_read_b64_tr_b16), each serving all row blocks
 //
-// Two row blocks per wave halve the LDS bytes read per flop: with one block per wave the four
-// waves would need the whole LDS bandwidth of the CU just to feed the matrix pipe at its peak.
+// The loop is a hand-ordered software pipeline: the scores of tile i + 1 run on the matrix pipe
+// under the exponentials of tile i, the products of tile i under the maxima and the score
+// transform of tile i + 1.  Interior tiles of a link take a branch-free ring step.
 // LDS rows are unpadded and swizzled (piece c of tile row r at position c ^ swz(r)), see
 // va_mfma_stream.hip.  The query tile is rotated by all 256 threads, one row block of every wave
 // (128 rows) at a time, into the two ring buffers that are not yet in use.
 #include <hip/hip_runtime.h>
-
-#include <type_traits>
 
 #include "va_internal.h"
 #include "va_launch.h"
