@@ -242,41 +242,73 @@ constexpr int kAnyInFlight = 63;  // vmcnt(63): no wait on vector memory at all
 // `lds_base + 16 l` (lds_base is wave-uniform and travels in M0).  Written as assembly on purpose:
 // when the compiler sees such a load it makes every later LDS read wait for ALL of them
 // (it cannot tell the ring's buffers apart), which would serialise the ring.  Completion is
-// tracked by hand instead, with the vmcnt values of ring_barrier.
+// tracked by hand instead, with the vmcnt values of ring_barrier.  M0 is a reserved register the
+// compiler manages itself and cannot be named as a clobber, so every statement puts back the value
+// it found: a value the compiler keeps live in M0 across the statement stays intact.
 __device__ __forceinline__ void load_to_lds(const void* src, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base)
-               : "memory");  // M0 is scratch for the compiler too: it sets it right before each use of its own
+  uint32_t saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, off\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(src), "s"(lds_base)
+      : "memory");
 }
 // The same with a wave-uniform base address and a 32-bit per-lane byte offset (no vector ALU work
 // to form 64-bit addresses).
 __device__ __forceinline__ void load_to_lds(const void* base, uint32_t lane_offset, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base),
-               "s"(lds_base)
-               : "memory");
+  uint32_t saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(lane_offset), "s"(base), "s"(lds_base)
+      : "memory");
 }
-// Up to four such loads behind ONE setting of M0: the instruction's immediate offset is added to
-// the pool address AND to the LDS address, so load u of a group lands 1024 u bytes further on when
-// its per-lane offset has had 1024 u taken off beforehand (grouped_lane_offset).  Two scalar
-// instructions per group instead of three per load.
+// Two loads of per-lane addresses behind ONE setting of M0, the second landing 1024 bytes after
+// the first: the instruction's immediate offset is added to the pool address AND to the LDS
+// address, so the caller passes the second address with 1024 taken off.
+__device__ __forceinline__ void load_pair_to_lds(const void* src0, const void* src1_minus_1024, uint32_t lds_base) {
+  uint32_t saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, off\n\t"
+      "global_load_lds_dwordx4 %2, off offset:1024\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(src0), "v"(src1_minus_1024), "s"(lds_base)
+      : "memory");
+}
+// Up to four loads of "uniform base + per-lane offset" behind one setting of M0: load u of a group
+// lands 1024 u bytes further on when its per-lane offset has had 1024 u taken off beforehand
+// (grouped_lane_offset).
 __device__ __forceinline__ uint32_t grouped_lane_offset(uint32_t lane_offset, int u) { return lane_offset - 1024u * (u % 4); }
 template <int kCount>
 __device__ __forceinline__ void load_group_to_lds(const void* base, const uint32_t* adjusted_offsets, uint32_t lds_base) {
   static_assert(kCount == 1 || kCount == 2 || kCount == 4, "loads per group");
+  uint32_t saved;
   if constexpr (kCount == 4) {
     asm volatile(
-        "s_mov_b32 m0, %5\n\ts_nop 0\n\t"
-        "global_load_lds_dwordx4 %0, %4\n\t"
-        "global_load_lds_dwordx4 %1, %4 offset:1024\n\t"
-        "global_load_lds_dwordx4 %2, %4 offset:2048\n\t"
-        "global_load_lds_dwordx4 %3, %4 offset:3072" ::"v"(adjusted_offsets[0]),
-        "v"(adjusted_offsets[1]), "v"(adjusted_offsets[2]), "v"(adjusted_offsets[3]), "s"(base), "s"(lds_base)
+        "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %6\n\ts_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, %5\n\t"
+        "global_load_lds_dwordx4 %2, %5 offset:1024\n\t"
+        "global_load_lds_dwordx4 %3, %5 offset:2048\n\t"
+        "global_load_lds_dwordx4 %4, %5 offset:3072\n\t"
+        "s_mov_b32 m0, %0"
+        : "=&s"(saved)
+        : "v"(adjusted_offsets[0]), "v"(adjusted_offsets[1]), "v"(adjusted_offsets[2]), "v"(adjusted_offsets[3]),
+          "s"(base), "s"(lds_base)
         : "memory");
   } else if constexpr (kCount == 2) {
     asm volatile(
-        "s_mov_b32 m0, %3\n\ts_nop 0\n\t"
-        "global_load_lds_dwordx4 %0, %2\n\t"
-        "global_load_lds_dwordx4 %1, %2 offset:1024" ::"v"(adjusted_offsets[0]),
-        "v"(adjusted_offsets[1]), "s"(base), "s"(lds_base)
+        "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %4\n\ts_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, %3\n\t"
+        "global_load_lds_dwordx4 %2, %3 offset:1024\n\t"
+        "s_mov_b32 m0, %0"
+        : "=&s"(saved)
+        : "v"(adjusted_offsets[0]), "v"(adjusted_offsets[1]), "s"(base), "s"(lds_base)
         : "memory");
   } else {
     load_to_lds(base, adjusted_offsets[0], lds_base);

@@ -66,16 +66,6 @@ __device__ __forceinline__ int swz(int r) {
   return (r >> 1) & 7;
 }
 
-#if VA_STREAM_TIMELINE  // experiment builds: per-workgroup start, set-up end, loop end, end, hardware id
-__device__ unsigned long long va_debug_times[8 * 16384];
-extern "C" __attribute__((visibility("default"))) int va_debug_read(void* host, size_t bytes) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(va_debug_times), bytes);
-}
-#define VA_STAMP(k) \
-  if (threadIdx.x == 0 && blockIdx.x < 16384) va_debug_times[8 * blockIdx.x + (k)] = wall_clock64();
-#else
-#define VA_STAMP(k)
-#endif
 
 template <typename E, int kD>
 __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void attn_stream_kernel(AttnArgs a) {
@@ -92,12 +82,6 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
   const int G = a.num_q_heads / a.num_kv_heads;
   const int n_q = item[VA_I_N_Q];
   if (n_q == 0) return;  // padding item: keeps the launch order aligned with the die round-robin
-  VA_STAMP(0)
-#if VA_STREAM_TIMELINE
-  if (threadIdx.x == 0 && blockIdx.x < 16384)
-    va_debug_times[8 * blockIdx.x + 4] = __builtin_amdgcn_s_getreg(4 | (31 << 11)) |
-                                         ((unsigned long long)__builtin_amdgcn_s_getreg(20 | (31 << 11)) << 32);
-#endif
   const int part_base = item[VA_I_PART_BASE];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -232,7 +216,6 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) qf[s] = q_stage[j * kChunks + ((4 * s + kg) ^ swz<kD>(j))];
     ring_barrier<kAnyInFlight>();  // the staging buffer may be refilled now
-    VA_STAMP(1)
 
     // ---- the tile loop, once per page-table kind so neither carries the other's branches ----
     auto stream = [&](auto uniform_tag) __attribute__((always_inline)) {
@@ -320,7 +303,6 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     }
   }
 
-  VA_STAMP(2)
   // row sums live spread over the four contraction groups
   l_run += __shfl_xor(l_run, 16, kWave);
   l_run += __shfl_xor(l_run, 32, kWave);
@@ -365,7 +347,6 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
       }
     }
   }
-  VA_STAMP(3)
 }
 
 template <typename E, int kD>

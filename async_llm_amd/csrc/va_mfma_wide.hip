@@ -357,11 +357,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     // wave makes every step exactly once, in order; a step is made just before tile k is first
     // needed (its K, for the scores computed one iteration ahead).
     constexpr float kRaise = 14.f;
-#if VA_WIDE_EXPERIMENT == 1  // ring only
-    const int n_vis = 0;
-#else
     const int n_vis = t_wave > tok_begin ? min(n_tiles, (t_wave - tok_begin + kWideTokens - 1) / kWideTokens) : 0;
-#endif
     int next_step = 0;
     // The pool row of the tile a step requests is looked up a whole step earlier (a scalar load whose
     // result is not touched before the next step): its latency never shows.
@@ -382,9 +378,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       } else {
         ring_barrier<0>();
       }
-#if VA_WIDE_EXPERIMENT != 5  // 5: computation only
       if (refill) issue(k + kWideAhead, row);
-#endif
     };
 
     // The same step for the steady part of a link (uniform pages; the requested tile and the one
@@ -398,9 +392,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       const int zero = ring_barrier_zero<(kWideAhead - 1) * kL>();
       const uint32_t dst = wave_lds + ring_slot(k + kWideAhead) * Sh::kBufferBytes;
       const char* base = wave_pool + row * row_bytes;
-#if VA_WIDE_EXPERIMENT != 5
       issue_plain(base, dst);
-#endif
       row_ahead = ((long long)(page + zero) << p_shift) + (t & (P - 1));
     };
     // iterations [1, i_steady_end) may take it: tiles i + 1 + kWideAhead and i + 2 + kWideAhead are plain,

@@ -181,6 +181,29 @@ class SharedCacheAttention:
         self._workspace: Optional[torch.Tensor] = None
         self._workspace_prepared = False
         self._plan_scratch = np.empty(1 << 16, dtype=np.int32)  # host scratch of the planner, grown on demand
+        self._checked_layers = set()
+        self._check_pool_layout()
+
+    def _check_pool_layout(self, layer_id: int = 0) -> None:
+        """``forward`` writes new K/V rows into ``k_cache(layer)`` / ``v_cache(layer)`` itself (the key
+        rotation is fused into the store) instead of calling ``kv_cache.store_kv`` as the reference
+        does (``attention.py:649``).  That is only the same thing for a pool that is a plain
+        ``[num_pages, page_size, kv_heads, head_dim]`` array of the op's dtype, so a pool of any other
+        layout is refused -- when the op is built, and again for every layer it stores into -- rather
+        than silently written wrongly.  A planner-only stand-in without layers (the reference's
+        planner tests pass a bare namespace) has nothing to check."""
+        want = (self.page_size, self.num_kv_heads, self.head_dim)
+        for name in ("k_cache", "v_cache"):
+            getter = getattr(self.kv_cache, name, None)
+            layer = getter(layer_id) if callable(getter) else None
+            if layer is None:
+                continue
+            if layer.dim() != 4 or tuple(layer.shape[1:]) != want:
+                raise ValueError(f"kv_cache.{name}({layer_id}) must be [num_pages, {want[0]}, {want[1]}, {want[2]}], "
+                                 f"got {tuple(layer.shape)}")
+            if layer.dtype != self.dtype or not layer.is_contiguous():
+                raise ValueError(f"kv_cache.{name}({layer_id}) must be a contiguous {self.dtype} tensor, got "
+                                 f"{layer.dtype}, contiguous={layer.is_contiguous()}")
 
     # ------------------------------------------------------------------
     # rotation
@@ -598,7 +621,9 @@ class SharedCacheAttention:
             v2 = v2.contiguous()
         k_pool = self.kv_cache.k_cache(layer_id)
         v_pool = self.kv_cache.v_cache(layer_id)
-        assert k_pool.is_contiguous() and v_pool.is_contiguous(), "pool layers must be contiguous"
+        if layer_id not in self._checked_layers:
+            self._check_pool_layout(layer_id)
+            self._checked_layers.add(layer_id)
         out_loc = batch.out_loc
         assert out_loc.dtype in (torch.int32, torch.int64) and out_loc.numel() == W
         out_loc = out_loc.contiguous()

@@ -18,7 +18,6 @@ Accounting (per forward, one layer):
 
 from __future__ import annotations
 
-import os
 from dataclasses import dataclass, field
 from types import SimpleNamespace
 from typing import Dict, List, Optional
@@ -64,8 +63,6 @@ class _Pages:
 
     def __init__(self, num_pages: int, page_size: int, gen: torch.Generator):
         self.order = torch.randperm(num_pages, generator=gen).tolist()
-        if os.environ.get("VIEWATTN_SEQUENTIAL_PAGES"):  # experiment: identity page table
-            self.order = list(range(num_pages))
         self.page_size = page_size
         self.used = 0
 

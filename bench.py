@@ -1,19 +1,23 @@
 """Benchmark of cache-view attention on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload batched_decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 A step is one ``SharedCacheAttention.forward`` of one layer (fused key
-rotate + KV store, attention, merge) over the batched bf16 decode
-configuration: 64 requests, 16 q / 4 kv heads, head_dim 256, page size 16,
-every view = one shared 8192-token block + 1-3 private blocks of 256..8192
-tokens.  Inputs are resident in HBM before the timed region; successive steps
+rotate + KV store, attention, merge).  Without ``--workload`` the line is the
+batched bf16 decode configuration (64 requests, 16 q / 4 kv heads, head_dim 256,
+page size 16, every view = one shared 8192-token block + 1-3 private blocks of
+256..8192 tokens) and carries, under ``configs``, the same measurements for the
+view-conditioned prefill, the mixed continuous batch, the long-context mRoPE
+decode and the fp32 plumbing case; with ``--workload`` only that workload is
+measured.  Inputs are resident in HBM before the timed region; successive steps
 rotate over several copies of the KV pool so the 256 MB last-level cache cannot
 hold the working set.  Prints ONE JSON line.
 
-``value`` is algorithmic GB/s: compulsory bytes of a step (each distinct block
-counted once, see ``async_llm_amd.workloads``) divided by the wall time per
-step.  ``roofline`` prices the attention kernel alone, timed with HIP events on
-the stream it is launched on.  ``cpu_baseline`` times the CPU oracle (torch on
+``value`` is algorithmic GB/s (decode, mixed) or TFLOP/s (prefill): compulsory
+bytes of a step (each distinct block counted once) or flops of the visible
+(row, key) pairs, see ``async_llm_amd.workloads``, divided by the wall time per
+step.  ``roofline`` prices the attention launches alone, timed with HIP events on
+the stream they are launched on.  ``cpu_baseline`` times the CPU oracle (torch on
 the host cores) on a bounded sample of the same workload.
 """
 
@@ -35,11 +39,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes one launch (attention + merge) moves at the default sizes, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs of this script scaled by the readings of --workload
 # copy_calibration (bytes = 2 KiB x FETCH_SIZE + 1 KiB x WRITE_SIZE); the summaries are in
-# profiles/.  A counter run cannot be made from inside the timed process, so the figure is
-# carried here and only reported for the configuration it was measured on.
-MEASURED_TRAFFIC_BYTES = {
-    ("batched_decode", "mfma"): (2_319_602 + 17_963 + 17_893 + 512) * 1024,
-    ("view_prefill", "mfma"): (2 * 7_356_834 + 131_084) * 1024,
+# profiles/.  A counter run cannot be made from inside the timed process, so the figures are
+# carried here together with the digest of the kernel sources they were measured on
+# (csrc_digest()), and are reported only while that digest is the one of the sources in the tree.
+MEASURED_TRAFFIC = {
 }
 
 
@@ -48,14 +51,13 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default: about a second of GPU time)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default: steps / 10)")
-    ap.add_argument("--workload", default="batched_decode",
+    ap.add_argument("--workload", default=None,
                     choices=["batched_decode", "mrope_decode", "view_prefill", "plumbing_decode", "mixed_batch",
                              "copy_calibration", "block_merge"])
     ap.add_argument("--layers", type=int, default=4, help="copies of the KV pool rotated over")
     ap.add_argument("--kernel", default=None, choices=[None, "auto", "generic", "mfma"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=0, help="requests in the CPU sample (0 = pick by size)")
-    ap.add_argument("--extra", action="store_true", help="also time the prefill configuration")
     return ap.parse_args()
 
 
@@ -96,7 +98,10 @@ def time_attention_kernel(wl, steps, warmup, layers):
 
 def cpu_baseline(wl, sample):
     """The CPU oracle on the first ``sample`` requests of the workload (same
-    blocks, same inputs): rotate+store, per-segment attention, merge."""
+    blocks, same inputs): rotate+store, per-segment attention, merge.  A mixed
+    batch takes its first ``sample`` decode rows and its first prefill chunk.
+    Returns (seconds per pass, compulsory bytes of the sample, flops of the
+    sample, cores, description, timed passes)."""
     import torch
 
     from async_llm_amd.shared_cache import WorkerGroup
@@ -109,8 +114,12 @@ def cpu_baseline(wl, sample):
     torch.set_num_threads(cores)
     rope = oracle_rope(op, wl.theta)
     k_cpu, v_cpu = wl.pool.k_cache(0).cpu(), wl.pool.v_cache(0).cpu()
-    if wl.mode == "decode":
-        W = wl.group.num_workers
+    item = wl.q.element_size()
+    b_tok = 2 * Hkv * D * item
+    runs, what = [], []
+    distinct, pairs = {}, 0
+    W = wl.group.num_workers if wl.group is not None else 0
+    if wl.mode in ("decode", "mixed"):
         n = min(W, sample)
         group = WorkerGroup(wl.group.workers[:n])
         pending = {id(b): wl.pending[id(b)] for b in group.write_to}
@@ -120,42 +129,56 @@ def cpu_baseline(wl, sample):
         pos = wl.batch.positions.cpu()[:n]
         logical = sum(plan.seq_lens) + len(plan.aux_slots)
 
-        def run():
+        def run_decode():
             k_rot = rope.rotate(k.view(n, Hkv, D), pos)
             O.store_kv(k_cpu.view(-1, Hkv * D), v_cpu.view(-1, Hkv * D), slots, k_rot.reshape(n, -1), v)
             return O.forward_decode(plan, q.view(n, Hq, D), k_cpu, v_cpu, rope)[0]
 
-        # compulsory bytes of the sample: distinct blocks once
-        distinct = {}
-        for view in group.cache_structure:
+        runs.append(run_decode)
+        for view in group.cache_structure:  # compulsory bytes of the sample: distinct blocks once
             for b in view:
                 distinct[id(b)] = b.num_tokens + (1 if id(b) in pending else 0)
-        sample_bytes = 2 * Hkv * D * q.element_size() * sum(distinct.values())
-        what = f"first {n} of {W} requests ({logical} logical KV tokens)"
-    else:
-        n = min(len(wl.specs), sample)
+        pairs += logical
+        what.append(f"first {n} of {W} decode requests ({logical} logical KV tokens)")
+    if wl.mode in ("prefill", "mixed"):
+        n = min(len(wl.specs), sample if wl.mode == "prefill" else 1)
         specs = wl.specs[:n]
-        plan = oracle_prefill_plan(specs, P)
-        rows = plan.num_rows
-        q, k, v = wl.q.cpu()[:rows], wl.k.cpu()[:rows], wl.v.cpu()[:rows]
-        pos = wl.batch.positions.cpu()[:rows]
-        out_loc = wl.batch.out_loc.cpu()[:rows]
+        plan_p = oracle_prefill_plan(specs, P)
+        rows = plan_p.num_rows
+        qp, kp, vp = wl.q.cpu()[W:W + rows], wl.k.cpu()[W:W + rows], wl.v.cpu()[W:W + rows]
+        pos_p = wl.batch.positions.cpu()[W:W + rows]
+        out_loc = wl.batch.out_loc.cpu()[W:W + rows]
 
-        def run():
-            k_rot = rope.rotate(k.view(rows, Hkv, D), pos)
-            O.store_kv(k_cpu.view(-1, Hkv * D), v_cpu.view(-1, Hkv * D), out_loc, k_rot.reshape(rows, -1), v)
-            return O.forward_prefill_batch(plan, q.view(rows, Hq, D), k_cpu, v_cpu, rope)[0]
+        def run_prefill():
+            k_rot = rope.rotate(kp.view(rows, Hkv, D), pos_p)
+            O.store_kv(k_cpu.view(-1, Hkv * D), v_cpu.view(-1, Hkv * D), out_loc, k_rot.reshape(rows, -1), vp)
+            return O.forward_prefill_batch(plan_p, qp.view(rows, Hq, D), k_cpu, v_cpu, rope)[0]
 
-        sample_bytes = None
-        what = f"first {n} of {len(wl.specs)} requests"
+        runs.append(run_prefill)
+        for s in specs:
+            for b in s.context:
+                distinct[id(b)] = b.num_tokens
+            distinct[("own", id(s))] = s.self_prefix_len + s.num_new
+            before = sum(b.num_tokens for b in s.context) + s.self_prefix_len
+            pairs += s.num_new * before + s.num_new * (s.num_new + 1) // 2
+        what.append(f"first {n} of {len(wl.specs)} prefill requests ({rows} new tokens)")
+
+    def run():
+        for r in runs:
+            r()
+
+    t0 = time.perf_counter()
     run()
-    reps = []
-    for _ in range(3):
+    first = time.perf_counter() - t0
+    reps = 3 if first < 4.0 else 1  # a long sample is timed once more after this warm-up pass
+    times = []
+    for _ in range(reps):
         t0 = time.perf_counter()
         run()
-        reps.append(time.perf_counter() - t0)
-    t = sorted(reps)[1]
-    return t, sample_bytes, cores, what, n
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[len(times) // 2]
+    sample_bytes = b_tok * sum(distinct.values())
+    return t, sample_bytes, 4 * D * Hq * pairs, cores, " + ".join(what), reps
 
 
 def copy_calibration(dev, steps):
@@ -279,6 +302,138 @@ def block_merge(dev, steps, warmup, layers, cpu):
     return 0
 
 
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def csrc_digest() -> str:
+    """Digest of the kernel and planner sources: a traffic figure measured with rocprofv3 is only
+    reported while the sources it was measured on are the ones that are running."""
+    import hashlib
+
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "async_llm_amd", "csrc")
+    for name in sorted(os.listdir(src)):
+        with open(os.path.join(src, name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
+
+
+def host_prepare_ms(wl, reps=20):
+    """Median wall time of planning the step again on the host (``prepare`` /
+    ``prepare_prefill_batch`` / ``prepare_mixed``), uploads included."""
+    import torch
+
+    op = wl.op
+    if wl.mode == "decode":
+        call = lambda: op.prepare(wl.group, wl.pending, wl.new_token_slots)
+    elif wl.mode == "prefill":
+        call = lambda: op.prepare_prefill_batch(wl.specs)
+    else:
+        call = lambda: op.prepare_mixed(wl.group, wl.pending, wl.new_token_slots, wl.specs)
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        meta = call()
+        times.append((time.perf_counter() - t0) * 1e3)
+        del meta
+    torch.cuda.synchronize()
+    return sorted(times)[len(times) // 2]
+
+
+def measure(wl, steps, warmup, layers, cpu_sample, with_cpu, traffic_ok):
+    """Time one workload: whole steps by the wall clock, the attention launches alone with HIP
+    events, the host planner, and the CPU oracle on a bounded sample.  Returns the fields of a
+    bench line (``steps`` / ``warmup`` as used)."""
+    import torch
+
+    # The shader clock idles at ~0.15 GHz and takes some milliseconds of load to reach its working
+    # frequency: run the step untimed for a while first (not counted in W or K), so that a short
+    # K measures the kernels and not the ramp.
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < 0.2:
+        for i in range(8):
+            wl.forward(i % layers)
+        torch.cuda.synchronize()
+    if steps is None:  # about a second of steps
+        t0 = time.perf_counter()
+        for i in range(8):
+            wl.forward(i % layers)
+        torch.cuda.synchronize()
+        steps = max(20, min(2000, int(8 / (time.perf_counter() - t0))))
+    if warmup is None:
+        warmup = max(4, steps // 10)
+
+    # whole step (store + attention + merge), wall clock around K steps
+    for i in range(warmup):
+        wl.forward(i % layers)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        wl.forward(i % layers)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+
+    kern_avg_ms, kern_med_ms = time_attention_kernel(wl, steps, warmup, layers)
+    counts = wl.meta.launch.counts
+    family = {1: "generic", 2: "mfma"}.get(counts.kernel)
+    decode = wl.mode in ("decode", "mixed")  # the mixed batch is priced against HBM, its binding roof
+    if decode:
+        metric, unit = "view_attention_decode_hbm_gbps", "GB/s"
+        value = wl.alg_bytes / (ms_per_step * 1e-3) / 1e9
+        achieved = wl.alg_bytes / (kern_avg_ms * 1e-3) / 1e9
+        roof = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None)
+    else:
+        metric, unit = "view_attention_prefill_mfma_tflops", "TFLOP/s"
+        value = wl.alg_flops / (ms_per_step * 1e-3) / 1e12
+        achieved = wl.alg_flops / (kern_avg_ms * 1e-3) / 1e12
+        roof = dict(bound="mfma", achieved=round(achieved, 2), peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
+                    frac=round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), traffic=None)
+    measured = MEASURED_TRAFFIC.get((wl.name, family))
+    if traffic_ok and measured and measured["csrc"] == csrc_digest():
+        roof["traffic"] = measured["bytes"]
+        roof["traffic_source"] = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, sources " + measured["csrc"]
+    roof.update(kernel="attention launch (all work items) + merge", kernel_ms_avg=round(kern_avg_ms, 4),
+                kernel_ms_median=round(kern_med_ms, 4))
+    dtype = (str(wl.op.dtype).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32")
+             .replace("float16", "f16"))
+    line = {
+        "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": {"workload": wl.name, "rows": wl.info.get("rows"), "q_heads": wl.op.num_qo_heads,
+                   "kv_heads": wl.op.num_kv_heads, "head_dim": wl.op.head_dim, "page_size": wl.op.page_size,
+                   "kv_pool_copies": layers, "alg_bytes": wl.alg_bytes, "logical_bytes": wl.logical_bytes,
+                   "alg_flops": wl.alg_flops, "kernel_family": family, "work_items": counts.n_items,
+                   "wide_items": counts.n_wide_items, "kv_chunk": counts.kv_chunk, "q_tile": counts.q_tile,
+                   "partials": counts.n_partials, "host_prepare_ms": round(host_prepare_ms(wl), 3)},
+        "roofline": roof,
+    }
+    if with_cpu:
+        sample = cpu_sample or {"decode": 64, "prefill": 1, "mixed": 8}[wl.mode]
+        t_cpu, sample_bytes, sample_flops, cores, what, reps = cpu_baseline(wl, sample)
+        if decode:
+            cpu_value, cpu_unit = sample_bytes / t_cpu / 1e9, "GB/s"
+        else:
+            cpu_value, cpu_unit = sample_flops / t_cpu / 1e12, "TFLOP/s"
+        line["cpu_baseline"] = {"value": round(cpu_value, 4), "unit": cpu_unit, "cores": cores,
+                                "cpu_model": cpu_model(), "kind": "port",
+                                "sample": what + f", {t_cpu:.2f} s per pass, torch CPU oracle, "
+                                + ("median of 3" if reps == 3 else "one pass after one warm-up" if reps == 1 else f"{reps} passes")}
+    return line
+
+
+SECONDARY = ("view_prefill", "mixed_batch", "mrope_decode", "plumbing_decode")
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -299,80 +454,31 @@ def main() -> int:
         return copy_calibration(dev, args.steps)
     if args.workload == "block_merge":
         return block_merge(dev, args.steps, args.warmup, args.layers, not args.no_cpu_baseline)
-    wl = build_workload(args.workload, dev, args.layers, args.kernel)
-    layers = args.layers
-
-    # The shader clock idles at ~0.15 GHz and takes some milliseconds of load to reach its working
-    # frequency: run the step untimed for a while first (not counted in W or K), so that a short
-    # K measures the kernels and not the ramp.
-    t_ramp = time.perf_counter()
-    while time.perf_counter() - t_ramp < 0.2:
-        for i in range(8):
-            wl.forward(i % layers)
-        torch.cuda.synchronize()
-    if args.steps is None:  # about a second of steps
-        t0 = time.perf_counter()
-        for i in range(8):
-            wl.forward(i % layers)
-        torch.cuda.synchronize()
-        args.steps = max(20, min(2000, int(8 / (time.perf_counter() - t0))))
-    if args.warmup is None:
-        args.warmup = max(4, args.steps // 10)
-
-    # whole step (store + attention + merge), wall clock around K steps
-    for i in range(args.warmup):
-        wl.forward(i % layers)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        wl.forward(i % layers)
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    kern_avg_ms, kern_med_ms = time_attention_kernel(wl, args.steps, args.warmup, layers)
-    counts = wl.meta.launch.counts
-    decode = wl.mode in ("decode", "mixed")  # the mixed batch is priced against HBM, its binding roof
-    if decode:
-        metric, unit = "view_attention_decode_hbm_gbps", "GB/s"
-        value = wl.alg_bytes / (ms_per_step * 1e-3) / 1e9
-        achieved = wl.alg_bytes / (kern_avg_ms * 1e-3) / 1e9
-        roof = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None)
-    else:
-        metric, unit = "view_attention_prefill_mfma_tflops", "TFLOP/s"
-        value = wl.alg_flops / (ms_per_step * 1e-3) / 1e12
-        achieved = wl.alg_flops / (kern_avg_ms * 1e-3) / 1e12
-        roof = dict(bound="mfma", achieved=round(achieved, 2), peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
-                    frac=round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), traffic=None)
-    if args.layers == 4 and not os.environ.get("VIEWATTN_PLAN"):
-        roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((wl.name, {1: "generic", 2: "mfma"}.get(counts.kernel)))
-    roof.update(kernel="attention launch (all work items) + merge", kernel_ms_avg=round(kern_avg_ms, 4),
-                kernel_ms_median=round(kern_med_ms, 4))
-
-    line = {
-        "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": str(wl.op.dtype).replace("torch.", "").replace("bfloat16", "bf16")
-        .replace("float32", "f32").replace("float16", "f16"),
-        "data": "synthetic",
-        "config": {"workload": wl.name, "rows": wl.info.get("rows"), "q_heads": wl.op.num_qo_heads,
-                   "kv_heads": wl.op.num_kv_heads, "head_dim": wl.op.head_dim, "page_size": wl.op.page_size,
-                   "kv_pool_copies": layers, "alg_bytes": wl.alg_bytes, "logical_bytes": wl.logical_bytes,
-                   "alg_flops": wl.alg_flops,
-                   "kernel_family": {1: "generic", 2: "mfma"}.get(counts.kernel), "work_items": counts.n_items,
-                   "kv_chunk": counts.kv_chunk, "q_tile": counts.q_tile, "partials": counts.n_partials},
-        "roofline": roof,
-    }
-    if not args.no_cpu_baseline:
-        sample = args.cpu_sample or (64 if decode else 2)
-        t_cpu, sample_bytes, cores, what, n = cpu_baseline(wl, sample)
-        if decode:
-            cpu_value, cpu_unit = sample_bytes / t_cpu / 1e9, "GB/s"
-        else:
-            per_req = wl.alg_flops / len(wl.specs)
-            cpu_value, cpu_unit = per_req * n / t_cpu / 1e12, "TFLOP/s"
-        line["cpu_baseline"] = {"value": round(cpu_value, 4), "unit": cpu_unit, "cores": cores, "kind": "port",
-                                "sample": what + f", {t_cpu:.2f} s per pass, torch CPU oracle, median of 3"}
+    # the default run reports every configuration: the batched decode as the line itself, the others
+    # under "configs"; naming a workload measures that one alone (what the profiler runs do)
+    everything = args.workload is None
+    name = args.workload or "batched_decode"
+    traffic_ok = args.layers == 4 and not os.environ.get("VIEWATTN_PLAN")
+    wl = build_workload(name, dev, args.layers, args.kernel)
+    line = measure(wl, args.steps, args.warmup, args.layers, args.cpu_sample, not args.no_cpu_baseline, traffic_ok)
+    del wl
+    if everything:
+        line["configs"] = {}
+        for other in SECONDARY:
+            torch.cuda.empty_cache()
+            layers = 1 if other == "plumbing_decode" else args.layers
+            wl = build_workload(other, dev, layers, args.kernel)
+            sub = measure(wl, None if other == "plumbing_decode" else max(20, args.steps or 20), None, layers, 0,
+                          not args.no_cpu_baseline, traffic_ok)
+            del wl
+            line["configs"][other] = {
+                "metric": sub["metric"], "value": sub["value"], "unit": sub["unit"], "dtype": sub["dtype"],
+                "steps": sub["steps"], "warmup": sub["warmup"], "ms_per_step": sub["ms_per_step"],
+                "alg_bytes": sub["config"]["alg_bytes"], "alg_flops": sub["config"]["alg_flops"],
+                "rows": sub["config"]["rows"], "work_items": sub["config"]["work_items"],
+                "wide_items": sub["config"]["wide_items"], "partials": sub["config"]["partials"],
+                "host_prepare_ms": sub["config"]["host_prepare_ms"], "roofline": sub["roofline"],
+                "cpu_baseline": sub.get("cpu_baseline")}
     print(json.dumps(line), flush=True)
     return 0
 

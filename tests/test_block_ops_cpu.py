@@ -151,7 +151,8 @@ def make_ops(page=4):
     from async_llm_amd.shared_cache import SharedCacheAttention
 
     cpu = torch.device("cpu")
-    pool = SimpleNamespace(k_cache=lambda layer: None, v_cache=lambda layer: None, num_layers=1)
+    layer = torch.zeros(8, page, 2, 16, dtype=torch.bfloat16)
+    pool = SimpleNamespace(k_cache=lambda _: layer, v_cache=lambda _: layer, num_layers=1)
     att = SharedCacheAttention(pool, torch.zeros(64, 16), 8, 2, 16, page, torch.bfloat16, cpu, rotary_dim=16)
     return BlockKVOps(pool, att, Alloc(page, 1))
 

@@ -133,3 +133,25 @@ def test_worker_group_rejections():
         WorkerGroup([ctx], cache_structure=[[prompt]])
     with pytest.raises(AssertionError):
         WorkerGroup()
+
+
+def test_op_refuses_a_pool_whose_layers_are_not_plain_paged_arrays():
+    """The op writes K/V rows into the pool itself (the reference calls ``kv_cache.store_kv``,
+    ``attention.py:649``), so the layout it assumes is checked when it is built."""
+    from types import SimpleNamespace
+
+    import pytest
+
+    from async_llm_amd.shared_cache import SharedCacheAttention
+
+    def build(layer, dtype=torch.bfloat16):
+        pool = SimpleNamespace(k_cache=lambda _: layer, v_cache=lambda _: layer)
+        return SharedCacheAttention(pool, torch.zeros(64, 16), 8, 2, 16, 4, dtype, torch.device("cpu"), rotary_dim=16)
+
+    build(torch.zeros(8, 4, 2, 16, dtype=torch.bfloat16))
+    with pytest.raises(ValueError, match="must be"):
+        build(torch.zeros(8, 2, 4, 16, dtype=torch.bfloat16))  # heads before tokens
+    with pytest.raises(ValueError, match="contiguous"):
+        build(torch.zeros(8, 4, 2, 32, dtype=torch.bfloat16)[..., :16])
+    with pytest.raises(ValueError, match="contiguous"):
+        build(torch.zeros(8, 4, 2, 16, dtype=torch.float16))

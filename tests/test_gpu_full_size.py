@@ -12,7 +12,6 @@ configurations, where an element-wise oracle run is too slow for a test:
   bit for bit and leaves the LSE alone.
 """
 
-import math
 import os
 
 import pytest
@@ -58,7 +57,54 @@ def test_mixed_batch_full_size_counts_every_visible_token_once():
     wl = workloads.mixed_batch(DEV, layers=1)  # configuration 4: 48 decode rows + 4 chunks of 512 in one launch
     out, lse = _zero_keys_unit_values(wl)
     assert torch.equal(out, torch.ones_like(out))
-    assert torch.isfinite(lse).all() and (lse > math.log(512)).all()  # every row sees at least the shared prompt
+    # decode rows see their whole view plus this step's token; row u of a chunk sees its context, the
+    # prefix of its own block and new tokens 0..u
+    want = [torch.tensor([sum(b.num_tokens for b in view) + 1 for view in wl.group.cache_structure],
+                         dtype=torch.float64)]
+    for s in wl.specs:
+        before = sum(b.num_tokens for b in s.context) + s.self_prefix_len
+        want.append(torch.arange(1, s.num_new + 1, dtype=torch.float64) + before)
+    want = torch.cat(want).log()[:, None].expand(-1, wl.op.num_qo_heads)
+    assert lse.shape == want.shape
+    assert torch.allclose(lse.double().cpu(), want, atol=1e-5, rtol=0), (lse.double().cpu() - want).abs().max()
+
+
+def test_mrope_decode_full_size_counts_every_token_once():
+    # configuration 5: 8 requests x 8 blocks x 16384 tokens; the only configuration whose pool byte
+    # offsets pass 2^31 (65 k pages of 32 KB per layer)
+    wl = workloads.mrope_decode(DEV, layers=1)
+    assert wl.pool.k_cache(0).numel() * wl.pool.k_cache(0).element_size() > 2 ** 31
+    out, lse = _zero_keys_unit_values(wl)
+    assert torch.equal(out, torch.ones_like(out))
+    tokens = torch.tensor([sum(b.num_tokens for b in view) + 1 for view in wl.group.cache_structure], dtype=torch.float64)
+    assert tokens.min() == 8 * 16384 + 1
+    want = tokens.log()[:, None].expand(-1, wl.op.num_qo_heads)
+    assert torch.allclose(lse.double().cpu(), want, atol=1e-5, rtol=0), (lse.double().cpu() - want).abs().max()
+
+
+def test_mrope_decode_full_size_reads_the_right_rows():
+    # zero keys make every row of V weigh the same, so the output is the mean of the value rows the
+    # view's page tables name.  Every value row holds the number of the 128 MB region of the pool it
+    # lives in (exact in bf16), so rows fetched through an offset folded to 32 bits (the pool is 4 GB
+    # per layer) come from other regions and move the mean.
+    wl = workloads.mrope_decode(DEV, layers=1)
+    k_pool, v_pool = wl.pool.k_cache(0), wl.pool.v_cache(0)
+    k_pool.zero_()
+    slots = torch.arange(v_pool.shape[0] * v_pool.shape[1], device=DEV)
+    tag = slots >> 16  # 65536 slots of 2 KB: region number, 0..16
+    v_pool.view(slots.numel(), -1).copy_(tag[:, None].to(v_pool.dtype).expand(-1, v_pool.shape[2] * v_pool.shape[3]))
+    v_new = torch.zeros_like(wl.v)
+    out, _ = wl.op.forward_with_lse(wl.q, torch.zeros_like(wl.k), v_new, 0, wl.batch)
+    P = wl.op.page_size
+    want = []
+    for w, view in enumerate(wl.group.cache_structure):
+        starts = torch.tensor([s for b in view for s in b.page_starts], dtype=torch.int64)
+        rows = (starts[:, None] + torch.arange(P)[None, :]).reshape(-1)
+        n = sum(b.num_tokens for b in view)
+        assert rows.numel() == n  # full pages; the appended token (value 0) lives in a pending page
+        want.append(tag.cpu()[rows].double().sum() / (n + 1))
+    want = torch.stack(want)[:, None].expand(-1, out.shape[1])
+    assert torch.allclose(out.double().cpu(), want, atol=0.0, rtol=6e-3), (out.double().cpu() - want).abs().max()
 
 
 @pytest.mark.parametrize("name", ["batched_decode", "view_prefill"])

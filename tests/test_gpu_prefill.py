@@ -218,3 +218,52 @@ def test_long_links_of_whole_pages(dtype, heads, rotary, mrope):
     assert first <= 200
     *_, meta = run_prefill_parity(op, cpu_pool, dev_pool, specs, 1e4, gen, scale=1.0 if heads[2] <= 64 else 0.5)
     assert meta.launch.counts.kernel == 2 and meta.launch.counts.n_wide_items > 0
+
+
+@pytest.mark.parametrize("spike", [13.0, 15.0, 40.0])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_wide_tiles_with_a_late_score_spike(D, dtype, spike):
+    """The wide kernel keeps a per-row reference maximum and raises it in the middle of a segment
+    only when a later tile exceeds it by more than 14 (log2 units).  Random N(0,1) scores never do,
+    so here single keys are planted whose score is ``spike`` log2 units for every query row: one in
+    an interior tile of a context block (the branch-free part of the walk) and one among the new
+    tokens (the masked tiles at the causal edge).  Only the dims past ``rotary_dim`` carry the
+    spike, so no rotation touches it.  13 stays just under the threshold (P = 2^13 must survive the
+    16-bit P operand), 15 is just over it; with 40 the other keys are random and the spike towers
+    over their running maximum."""
+    heads, page, rotary = (8, 2, D), 16, D // 2
+    random_keys = spike > 20
+    op, cpu_pool, dev_pool, gen = make_op_and_pool(DEV, dtype, heads, page, 96, 1e4, rotary_dim=rotary, seed=91,
+                                                   scale=1.0, kernel="auto", max_pos=2048)
+    a = spike * 2.0 / (D ** 0.5 * 1.4426950408889634)  # a * (D/2) / sqrt(D) * log2(e) == spike
+    if not random_keys:
+        for pool in (cpu_pool[0], dev_pool[0]):
+            pool.zero_()
+    context = CacheBlock(DEV, page)
+    context.grow_pages(torch.arange(0, 30) * page, 470)
+    planted = 8 * page + 5  # token 213 of the context block (pages are in order here)
+    for pool in (cpu_pool[0], dev_pool[0]):
+        pool.view(-1, heads[1], D)[planted, :, :rotary] = 0
+        pool.view(-1, heads[1], D)[planted, :, rotary:] = a
+    new_tokens, prefix = 200, 24
+    pages = torch.arange(40, 40 + -(-(prefix + new_tokens) // page), dtype=torch.int32) * page
+    specs = [PrefillSpec([context], pages, new_tokens, prefix)]
+
+    def mutate(q, k, v):
+        q.view(-1, heads[0], D)[:, :, rotary:] = 1.0
+        if not random_keys:
+            k.zero_()
+        k.view(-1, heads[1], D)[150, :, :rotary] = 0
+        k.view(-1, heads[1], D)[150, :, rotary:] = a
+
+    out, lse, exp_out, exp_lse, meta = run_prefill_parity(op, cpu_pool, dev_pool, specs, 1e4, gen, scale=1.0,
+                                                          mutate=mutate)
+    assert meta.launch.counts.n_wide_items > 0
+    if not random_keys:  # every other score is 0: the closed form of the row's logsumexp
+        seen = 470 + prefix + torch.arange(1, new_tokens + 1, dtype=torch.float64)
+        spikes = 1 + (torch.arange(new_tokens) >= 150).double()
+        a_stored = float(torch.tensor(a, dtype=dtype))  # the planted value as the pool holds it
+        want = (seen - spikes + spikes * torch.tensor(a_stored * (D / 2) / D ** 0.5, dtype=torch.float64).exp()).log()
+        got = lse.double().cpu()
+        assert torch.allclose(got, want[:, None].expand_as(got), atol=2e-2, rtol=0)

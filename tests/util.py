@@ -166,8 +166,9 @@ def oracle_prefill(op, cpu_pool, specs, theta, positions, mrope_positions, out_l
     return O.forward_prefill_batch(oracle_prefill_plan(specs, P), q.view(N, Hq, D), k_cpu, v_cpu, rope)
 
 
-def run_prefill_parity(op, cpu_pool, dev_pool, specs, theta, gen, scale=None):
-    """One batched prefill through the product op and through the oracle."""
+def run_prefill_parity(op, cpu_pool, dev_pool, specs, theta, gen, scale=None, mutate=None):
+    """One batched prefill through the product op and through the oracle.  ``mutate(q, k, v)`` may
+    edit the random input rows (CPU tensors) in place before either side sees them."""
     from types import SimpleNamespace
 
     dev = op.device
@@ -177,6 +178,8 @@ def run_prefill_parity(op, cpu_pool, dev_pool, specs, theta, gen, scale=None):
     assert torch.equal(meta.sub_loc.cpu(), oplan.sub_loc) and meta.pad_slot.tolist() == oplan.pad_slot
     N = meta.num_workers
     positions, mrope_positions, out_loc, q, k, v = prefill_inputs(op, specs, gen, scale)
+    if mutate is not None:
+        mutate(q, k, v)
     batch = SimpleNamespace(attn_metadata=meta, positions=positions.to(dev), out_loc=out_loc.to(dev),
                             mrope_positions=None if mrope_positions is None else mrope_positions.to(dev))
     out, lse = op.forward_with_lse(q.to(dev), k.to(dev), v.to(dev), 0, batch)
