@@ -141,8 +141,8 @@ def cpu_baseline(wl, sample):
         pairs += logical
         what.append(f"first {n} of {W} decode requests ({logical} logical KV tokens)")
     if wl.mode in ("prefill", "mixed"):
-        n = min(len(wl.specs), sample if wl.mode == "prefill" else 1)
-        specs = wl.specs[:n]
+        n_p = min(len(wl.specs), sample if wl.mode == "prefill" else 1)
+        specs = wl.specs[:n_p]
         plan_p = oracle_prefill_plan(specs, P)
         rows = plan_p.num_rows
         qp, kp, vp = wl.q.cpu()[W:W + rows], wl.k.cpu()[W:W + rows], wl.v.cpu()[W:W + rows]
@@ -161,7 +161,7 @@ def cpu_baseline(wl, sample):
             distinct[("own", id(s))] = s.self_prefix_len + s.num_new
             before = sum(b.num_tokens for b in s.context) + s.self_prefix_len
             pairs += s.num_new * before + s.num_new * (s.num_new + 1) // 2
-        what.append(f"first {n} of {len(wl.specs)} prefill requests ({rows} new tokens)")
+        what.append(f"first {n_p} of {len(wl.specs)} prefill requests ({rows} new tokens)")
 
     def run():
         for r in runs:
