@@ -5,6 +5,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/viewattn.h"
 #include "va_device.h"
@@ -496,13 +497,15 @@ extern "C" int va_store_kv_rope(const void* k_dev, const void* v_dev, int64_t k_
   return rc;
 }
 
-extern "C" int va_attention(const void* q_dev, int64_t q_row_stride, const void* k_pool_dev,
-                            const void* v_pool_dev, int64_t pool_row_stride, const int32_t* plan_dev,
-                            const int32_t* plan_header_host, const int32_t* kv_indices_dev,
-                            const int64_t* sub_worker_dev, const int64_t* sub_loc_dev,
-                            int64_t sub_loc_axis_stride, void* out_dev, float* lse_dev, int32_t lse_base2,
-                            void* workspace_dev, int64_t workspace_bytes, const VaShape* shape,
-                            const VaRope* rope, void* stream) {
+// Both attention entry points: `workspace_dev` is the caller's buffer (va_attention) or this
+// device's copy of the library's own scratch array (va_attention_static).
+static int attention_launches(const void* q_dev, int64_t q_row_stride, const void* k_pool_dev,
+                              const void* v_pool_dev, int64_t pool_row_stride, const int32_t* plan_dev,
+                              const int32_t* plan_header_host, const int32_t* kv_indices_dev,
+                              const int64_t* sub_worker_dev, const int64_t* sub_loc_dev,
+                              int64_t sub_loc_axis_stride, void* out_dev, float* lse_dev, int32_t lse_base2,
+                              void* workspace_dev, int64_t workspace_bytes, const VaShape* shape,
+                              const VaRope* rope, void* stream) {
   if (!shape || !plan_header_host || !plan_dev) return va_fail(VA_ERR_ARG, "null plan or shape");
   const int32_t* h = plan_header_host;
   if (h[VA_H_MAGIC] != VA_PLAN_MAGIC) return va_fail(VA_ERR_ARG, "plan header has no magic word");
@@ -574,4 +577,74 @@ extern "C" int va_attention(const void* q_dev, int64_t q_row_stride, const void*
     VA_DISPATCH_DTYPE(shape->dtype, rc = va::launch_merge<E>(m, n_rows, s));
   }
   return rc;
+}
+
+extern "C" int va_attention(const void* q_dev, int64_t q_row_stride, const void* k_pool_dev,
+                            const void* v_pool_dev, int64_t pool_row_stride, const int32_t* plan_dev,
+                            const int32_t* plan_header_host, const int32_t* kv_indices_dev,
+                            const int64_t* sub_worker_dev, const int64_t* sub_loc_dev,
+                            int64_t sub_loc_axis_stride, void* out_dev, float* lse_dev, int32_t lse_base2,
+                            void* workspace_dev, int64_t workspace_bytes, const VaShape* shape,
+                            const VaRope* rope, void* stream) {
+  return attention_launches(q_dev, q_row_stride, k_pool_dev, v_pool_dev, pool_row_stride, plan_dev, plan_header_host,
+                            kv_indices_dev, sub_worker_dev, sub_loc_dev, sub_loc_axis_stride, out_dev, lse_dev,
+                            lse_base2, workspace_dev, workspace_bytes, shape, rope, stream);
+}
+
+// ---------------------------------------------------------------------------
+// va_attention_static: the same launches over a scratch array the library owns
+// ---------------------------------------------------------------------------
+// Partial softmax states of rows served by several work items live here instead of in a caller's
+// workspace.  Every GPU the library runs on holds its own copy of the array, at its own address,
+// until the process ends.  In host code the array's name only stands for the symbol: the address
+// kernels may use is looked up once per device (hipGetSymbolAddress, with that device current) and
+// kept; nothing below passes the name itself to a kernel.
+static __device__ __align__(256) unsigned char scratch[VA_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of the current device's copy of `scratch` (NULL on failure, error recorded).
+void* static_scratch_of_current_device() {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess || device < 0 || device >= kMaxDevices) {
+    va_fail(VA_ERR_HIP, "static scratch: no current device (%s)", hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      va_fail(VA_ERR_HIP, "static scratch: hipGetSymbolAddress on device %d: %s", device, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[device] = ptr;
+  }
+  return g_scratch_ptr[device];
+}
+}  // namespace
+
+extern "C" int va_attention_static(const void* q_dev, int64_t q_row_stride, const void* k_pool_dev,
+                                   const void* v_pool_dev, int64_t pool_row_stride, const int32_t* plan_dev,
+                                   const int32_t* plan_header_host, const int32_t* kv_indices_dev,
+                                   const int64_t* sub_worker_dev, const int64_t* sub_loc_dev,
+                                   int64_t sub_loc_axis_stride, void* out_dev, float* lse_dev, int32_t lse_base2,
+                                   const VaShape* shape, const VaRope* rope, void* stream) {
+  if (!shape || !plan_header_host) return va_fail(VA_ERR_ARG, "null plan or shape");
+  if (plan_header_host[VA_H_MAGIC] != VA_PLAN_MAGIC) return va_fail(VA_ERR_ARG, "plan header has no magic word");
+  const int64_t need = va_workspace_bytes_for(plan_header_host[VA_H_N_PARTIALS], shape->num_q_heads, shape->head_dim);
+  if (need > (int64_t)VA_STATIC_SCRATCH_BYTES)
+    return va_fail(VA_ERR_CAPACITY,
+                   "va_attention_static: the plan's %d partial states need %lld bytes of scratch, the library's "
+                   "array holds %lld; use va_attention with a workspace of the caller's",
+                   plan_header_host[VA_H_N_PARTIALS], (long long)need, (long long)VA_STATIC_SCRATCH_BYTES);
+  void* ptr = static_scratch_of_current_device();
+  if (!ptr) return VA_ERR_HIP;
+  return attention_launches(q_dev, q_row_stride, k_pool_dev, v_pool_dev, pool_row_stride, plan_dev, plan_header_host,
+                            kv_indices_dev, sub_worker_dev, sub_loc_dev, sub_loc_axis_stride, out_dev, lse_dev,
+                            lse_base2, ptr, (int64_t)VA_STATIC_SCRATCH_BYTES, shape, rope, stream);
 }

@@ -22,6 +22,7 @@ VA_KERNEL_AUTO, VA_KERNEL_GENERIC, VA_KERNEL_MFMA = 0, 1, 2
 VA_SUB_CAUSAL, VA_SUB_SLOTS = 1, 2
 PLAN_HEADER_WORDS = 24
 VA_ERR_ARG, VA_ERR_CAPACITY = -1, -2
+STATIC_SCRATCH_BYTES = 32 << 20  # VA_STATIC_SCRATCH_BYTES: the array va_attention_static keeps on every GPU
 
 _DTYPES = {torch.float32: VA_F32, torch.float16: VA_F16, torch.bfloat16: VA_BF16}
 
@@ -37,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "va_plan_fixed_words",
     "va_plan_build_fixed",
     "va_attention",
+    "va_attention_static",
 )
 
 
@@ -155,6 +157,9 @@ def _load() -> C.CDLL:
     lib.va_attention.restype = C.c_int
     lib.va_attention.argtypes = [vp, i64, vp, vp, i64, vp, vp, vp, vp, vp, i64, vp, vp, i32, vp, i64,
                                  C.POINTER(VaShape), C.POINTER(VaRope), vp]
+    lib.va_attention_static.restype = C.c_int
+    lib.va_attention_static.argtypes = [vp, i64, vp, vp, i64, vp, vp, vp, vp, vp, i64, vp, vp, i32,
+                                        C.POINTER(VaShape), C.POINTER(VaRope), vp]
     return lib
 
 

@@ -633,9 +633,13 @@ class SharedCacheAttention:
             W, self._shape, self._rope_descriptor(), native.current_stream_ptr(self.device)))
 
     def attend(self, q: torch.Tensor, layer_id: int, meta: SharedCacheAttnMetadata,
-               return_lse: bool = False, lse_base2: bool = False):
+               return_lse: bool = False, lse_base2: bool = False, out: Optional[torch.Tensor] = None,
+               lse: Optional[torch.Tensor] = None, static_scratch: bool = False):
         """Run the planned attention over the pool as it is now; returns
-        ``out [rows, Hq*D]`` (and ``lse [rows, Hq]`` fp32 on request)."""
+        ``out [rows, Hq*D]`` (and ``lse [rows, Hq]`` fp32 on request).  With
+        ``static_scratch`` (and ``out`` / ``lse`` given) the call goes through
+        ``va_attention_static`` and allocates nothing: the partial states live in
+        the library's own per-GPU array, which bounds the plan's size."""
         native.require_device(q, "q")
         launch = meta.launch
         assert launch is not None, "metadata carries no launch plan"
@@ -644,20 +648,27 @@ class SharedCacheAttention:
         if q2.stride(-1) != 1:
             q2 = q2.contiguous()
         assert q2.shape[0] >= W and q2.dtype == self.dtype
-        out = torch.empty((W, Hq * D), dtype=self.dtype, device=self.device)
-        lse = torch.empty((W, Hq), dtype=torch.float32, device=self.device) if return_lse else None
+        if out is None:
+            out = torch.empty((W, Hq * D), dtype=self.dtype, device=self.device)
+        if lse is None and return_lse:
+            lse = torch.empty((W, Hq), dtype=torch.float32, device=self.device)
+        assert out.shape == (W, Hq * D) and out.dtype == self.dtype and out.is_contiguous()
+        assert lse is None or (lse.shape == (W, Hq) and lse.dtype == torch.float32 and lse.is_contiguous())
         k_pool = self.kv_cache.k_cache(layer_id)
         v_pool = self.kv_cache.v_cache(layer_id)
         sub_loc = meta.sub_loc
         axis_stride = sub_loc.stride(0) if sub_loc.dim() == 2 else 0
-        ws = launch.workspace
-        native.check(native.lib.va_attention(
-            q2.data_ptr(), q2.stride(0), k_pool.data_ptr(), v_pool.data_ptr(), self.num_kv_heads * D,
-            launch.blob.data_ptr(), launch.header.ctypes.data, launch.kv_indices.data_ptr(),
-            meta.sub_worker.data_ptr(), sub_loc.data_ptr(), axis_stride, out.data_ptr(),
-            None if lse is None else lse.data_ptr(), int(lse_base2),
-            None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(),
-            self._shape, self._rope_descriptor(), native.current_stream_ptr(self.device)))
+        head = (q2.data_ptr(), q2.stride(0), k_pool.data_ptr(), v_pool.data_ptr(), self.num_kv_heads * D,
+                launch.blob.data_ptr(), launch.header.ctypes.data, launch.kv_indices.data_ptr(),
+                meta.sub_worker.data_ptr(), sub_loc.data_ptr(), axis_stride, out.data_ptr(),
+                None if lse is None else lse.data_ptr(), int(lse_base2))
+        tail = (self._shape, self._rope_descriptor(), native.current_stream_ptr(self.device))
+        if static_scratch:
+            native.check(native.lib.va_attention_static(*head, *tail))
+        else:
+            ws = launch.workspace
+            native.check(native.lib.va_attention(*head, None if ws is None else ws.data_ptr(),
+                                                 0 if ws is None else ws.numel(), *tail))
         return (out, lse) if return_lse else out
 
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, layer_id: int, batch) -> torch.Tensor:

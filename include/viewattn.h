@@ -25,9 +25,10 @@
  * Conventions: every function returns 0 on success or a negative VA_ERR_*;
  * va_last_error() returns a thread-local message for the last failure.  All
  * pointers named *_dev are device pointers on the current HIP device; *_host are
- * host pointers.  The library allocates nothing and keeps no global state: the
- * caller owns every buffer (workspace included) and the stream.  `stream` is a
- * hipStream_t passed as void*.
+ * host pointers.  The library allocates nothing: the caller owns every buffer
+ * (workspace included) and the stream.  Its only state besides the last error
+ * message is the scratch array of va_attention_static (one copy per GPU).
+ * `stream` is a hipStream_t passed as void*.
  */
 #ifndef VIEWATTN_H
 #define VIEWATTN_H
@@ -287,6 +288,29 @@ VA_API int va_attention(const void* q_dev, int64_t q_row_stride, const void* k_p
                  int64_t sub_loc_axis_stride, void* out_dev, float* lse_dev, int32_t lse_base2,
                  void* workspace_dev, int64_t workspace_bytes, const VaShape* shape,
                  const VaRope* rope, void* stream);
+
+/*
+ * va_attention_static: va_attention for callers that cannot allocate or bring a
+ * workspace -- code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and
+ * results as va_attention without workspace_dev / workspace_bytes: the partial
+ * softmax states go to an array of VA_STATIC_SCRATCH_BYTES that the library
+ * holds on every GPU it runs on until the process ends.  The call allocates
+ * nothing (no hipMalloc / hipFree, no allocating library routine).  A plan whose
+ * partial states need more (n_partials * num_q_heads * (head_dim + 2) * 4 bytes)
+ * is rejected with VA_ERR_CAPACITY.  Every call on a GPU shares that GPU's
+ * array: nothing in it has to start at zero (each slot is written before the
+ * merge reads it), but calls that overlap on one GPU -- two streams, two
+ * threads -- race; run them in stream order.  The first call on a device looks
+ * up the array's device address; make it outside graph capture.
+ */
+#define VA_STATIC_SCRATCH_BYTES (32u << 20)
+VA_API int va_attention_static(const void* q_dev, int64_t q_row_stride, const void* k_pool_dev,
+                        const void* v_pool_dev, int64_t pool_row_stride, const int32_t* plan_dev,
+                        const int32_t* plan_header_host, const int32_t* kv_indices_dev,
+                        const int64_t* sub_worker_dev, const int64_t* sub_loc_dev,
+                        int64_t sub_loc_axis_stride, void* out_dev, float* lse_dev, int32_t lse_base2,
+                        const VaShape* shape, const VaRope* rope, void* stream);
 
 #ifdef __cplusplus
 }
