@@ -28,6 +28,11 @@ DEVICE_FLAGS = ["--offload-arch=gfx950", "--cuda-device-only",
                 # packed fp32 forms are kept out of the generated code
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HOST_FLAGS = ["--offload-arch=gfx950", "--cuda-host-only"]
+# Device flags of single sources.  The wide kernel may use all 512 registers of a lane, for which the
+# compiler gives every matrix product it selects an accumulator in the accumulation registers; its
+# score products are read by the vector ALU at once and want ordinary registers (the long-lived
+# output accumulators are pinned in accumulation registers by hand).
+SOURCE_DEVICE_FLAGS = {"va_mfma_wide.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def _run(cmd, verbose):
@@ -45,7 +50,8 @@ def _compile_one(hipcc, src, obj, extra, verbose):
     path = os.path.join(CSRC, src)
     if src.endswith(".hip"):
         fatbin = obj[:-2] + ".hipfb"
-        _run([hipcc, *COMMON_FLAGS, *DEVICE_FLAGS, *extra, "-c", path, "-o", fatbin], verbose)
+        _run([hipcc, *COMMON_FLAGS, *DEVICE_FLAGS, *SOURCE_DEVICE_FLAGS.get(src, []), *extra, "-c", path, "-o", fatbin],
+             verbose)
         _run([hipcc, *COMMON_FLAGS, *HOST_FLAGS, *extra, "-Xclang", "-fcuda-include-gpubinary", "-Xclang", fatbin,
               "-c", path, "-o", obj], verbose)
     else:

@@ -27,24 +27,17 @@ struct Mma<BF16> {
   }
   // Same product with the accumulator pinned in the accumulation registers (AGPRs).  Written as
   // assembly because the register allocator otherwise treats AGPRs as spill space for a long-lived
-  // accumulator and copies all of it to VGPRs and back around every tile.  The compiler cannot
-  // insert wait states for an instruction it does not see: the matrix pipe must not read an operand
-  // in the two wait states after a vector-ALU instruction wrote it, and ANY product can be preceded
-  // by such a write -- the transposed V fragment, the packed P, but also a register copy the
-  // allocator places in front of the statement (an operand parked in an AGPR is brought back with
-  // v_accvgpr_read right there).  Every product issued from assembly therefore carries its own
-  // `s_nop 1`; without it results depended on the register allocation of the build.  Callers wait
-  // (accumulator_fence) before reading an accumulator with anything but another product.
+  // accumulator and copies all of it to VGPRs and back around every tile.  Only the long-lived
+  // output accumulators are driven this way: nothing but further products touches them between
+  // the start of a work item and accumulator_fence(), which every other reader must call first
+  // (it carries the accumulators through, so no read can be moved in front of it).  The compiler
+  // cannot insert wait states for an instruction it does not see, and the matrix pipe must not
+  // read an operand in the two wait states after a vector-ALU instruction wrote it (the transposed
+  // V fragment, the packed P, or a register copy placed in front of the statement): every product
+  // issued from assembly therefore carries its own `s_nop 1`.  Products whose results the vector
+  // ALU reads next (the scores) go through run32, which the compiler sees and guards both ways.
   static __device__ __forceinline__ void run32_acc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-  }
-  // The same with the accumulator in ordinary vector registers (for results the vector ALU reads
-  // next, the scores); `first`: the sum starts from zero.
-  static __device__ __forceinline__ void run32_vacc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
-    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
-  }
-  static __device__ __forceinline__ void run32_vacc_first(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
-    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
   }
   template <typename A, typename B>
   static __device__ __forceinline__ va_f32x4 run(const A& a, const B& b, va_f32x4 c) {
@@ -72,12 +65,6 @@ struct Mma<F16> {
   }
   static __device__ __forceinline__ void run32_acc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-  }
-  static __device__ __forceinline__ void run32_vacc(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
-    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
-  }
-  static __device__ __forceinline__ void run32_vacc_first(const va_u32x4& a, const va_u32x4& b, va_f32x16& c) {
-    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
   }
   template <typename A, typename B>
   static __device__ __forceinline__ va_f32x4 run(const A& a, const B& b, va_f32x4 c) {
@@ -215,9 +202,29 @@ struct TableQueryUnit {
   }
 };
 
-// Wait until the matrix pipe has written the results of products issued from assembly
-// (run32_acc): 8 passes plus the write-back, 20 wait states.
-__device__ __forceinline__ void accumulator_fence() { asm volatile("s_nop 15\n\ts_nop 3" ::: "memory"); }
+// Wait until the matrix pipe has written the results of the products issued from assembly
+// (run32_acc) into the accumulators `o`, before anything but another product touches them.  A
+// 32x32x16 product runs for 8 passes of 4 clocks and its result needs 3 more wait states to reach
+// the register file (11 in all, whatever was issued before it has finished by then as the pipe
+// works in order); kAccumulatorWaitStates adds a margin.  The statement takes every accumulator as
+// an in-out operand: a later read depends on it and so cannot be scheduled in front of it, and
+// neither can a copy the register allocator makes for such a read.
+constexpr int kMfma32Passes = 8;
+constexpr int kAccumulatorWaitStates = kMfma32Passes + 3 + 4;
+static_assert(kAccumulatorWaitStates <= 16, "one s_nop holds at most 16 wait states");
+template <int kCount>
+__device__ __forceinline__ void accumulator_fence(va_f32x16* o) {
+  static_assert(kCount == 2 || kCount == 4 || kCount == 8, "accumulators per wave");
+  if constexpr (kCount == 8) {
+    asm volatile("s_nop %8"
+                 : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(o[4]), "+a"(o[5]), "+a"(o[6]), "+a"(o[7])
+                 : "n"(kAccumulatorWaitStates - 1));
+  } else if constexpr (kCount == 4) {
+    asm volatile("s_nop %4" : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]) : "n"(kAccumulatorWaitStates - 1));
+  } else {
+    asm volatile("s_nop %2" : "+a"(o[0]), "+a"(o[1]) : "n"(kAccumulatorWaitStates - 1));
+  }
+}
 
 // Workgroup barrier for the tile ring.  __syncthreads() carries a fence that waits for ALL
 // outstanding memory operations, which would drain the loads of the tiles still in flight; this

@@ -415,10 +415,12 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     auto score_step = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
       for (int b = 0; b < kB; ++b) {
+        // through the builtin: the compiler sees these products and keeps the wait states between
+        // them and the vector-ALU instructions that feed them or read their results
         if (s == 0) {
-          Mma<E>::run32_vacc_first(kf[s], qf[b][s], sc_next[b]);
+          sc_next[b] = Mma<E>::run32(kf[s], qf[b][s], va_f32x16{});
         } else {
-          Mma<E>::run32_vacc(kf[s], qf[b][s], sc_next[b]);
+          sc_next[b] = Mma<E>::run32(kf[s], qf[b][s], sc_next[b]);
         }
       }
     };
@@ -428,7 +430,6 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       read_k(0);
 #pragma unroll
       for (int s = 0; s < kSteps; ++s) score_step(s);
-      accumulator_fence();
 #pragma unroll
       for (int b = 0; b < kB; ++b) sc[b] = sc_next[b];
     }
@@ -587,7 +588,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       }
       if (resume) {
         // raise the references to this tile's maxima and rescale what was accumulated against the old ones
-        accumulator_fence();
+        accumulator_fence<kB * kDimTiles>(&o[0][0]);
 #pragma unroll
         for (int b = 0; b < kB; ++b) {
           const float m_new = fmaxf(m_ref[b], m_tile[b]);
@@ -610,7 +611,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     while (next_step < n_tiles) ring_step();  // tiles this wave does not see: keep in step with the others
   }
 
-  accumulator_fence();
+  accumulator_fence<kB * kDimTiles>(&o[0][0]);
   // ---- emit: accumulator reg r of dim tile t is dim 32t + (r/4)*8 + 4h + r%4 of the lane's row ----
 #pragma unroll
   for (int b = 0; b < kB; ++b) {
