@@ -29,6 +29,7 @@ struct AttnArgs {
   RopeDev rope;
   float scale_log2;  // log2(e) / sqrt(head_dim)
   const int32_t* qref_rows;  // sub_worker[qrefs[k]], precomputed by the planner
+  const int32_t* wide_slots;  // [n_wide_slots + 1]: the wide items each workgroup of the wide launch runs
 };
 
 struct MergeArgs {
@@ -47,9 +48,11 @@ struct MergeArgs {
 int make_rope(const VaRope* rope, int head_dim, RopeDev* out);
 
 // Matrix-core attention (launched from va_mfma.hip).
-// `n_wide` leading items are wide tiles (va_mfma_wide.hip), the rest narrow ones (va_mfma_stream.hip).
-int launch_mfma(const AttnArgs& a, int dtype, int n_items, int n_wide, int q_tile, hipStream_t stream);
-int launch_mfma_wide(const AttnArgs& a, int dtype, int n_items, hipStream_t stream);
+// `n_wide` leading items are wide tiles (va_mfma_wide.hip: `n_wide_slots` workgroups per kv head, each
+// running the items a.wide_slots gives it), the rest narrow ones (va_mfma_stream.hip).
+int launch_mfma(const AttnArgs& a, int dtype, int n_items, int n_wide, int n_wide_slots, int q_tile,
+                hipStream_t stream);
+int launch_mfma_wide(const AttnArgs& a, int dtype, int n_slots, hipStream_t stream);
 int launch_mfma_stream(const AttnArgs& a, int dtype, int n_items, hipStream_t stream);
 
 }  // namespace va

@@ -26,7 +26,8 @@ int va_mfma_wide_q_tile(int gqa, int head_dim) { return (head_dim == 256 ? 128 :
 
 namespace va {
 
-int launch_mfma(const AttnArgs& a_in, int dtype, int n_items, int n_wide, int q_tile, hipStream_t stream) {
+int launch_mfma(const AttnArgs& a_in, int dtype, int n_items, int n_wide, int n_wide_slots, int q_tile,
+                hipStream_t stream) {
   AttnArgs a = a_in;
   const int g = a.num_q_heads / a.num_kv_heads;
   if (!va_mfma_supported(dtype, a.head_dim, g))
@@ -37,8 +38,8 @@ int launch_mfma(const AttnArgs& a_in, int dtype, int n_items, int n_wide, int q_
     return va_fail(VA_ERR_ARG, "matrix-core path needs 16-byte aligned rows");
   // the streaming kernel addresses a tile's rows with 32-bit byte offsets from its first row
   if (a.pool_row_stride * 2 * 16 > 0x7fffffffLL) return va_fail(VA_ERR_ARG, "pool rows too far apart");
-  if (n_wide > 0) {
-    const int rc = launch_mfma_wide(a, dtype, n_wide, stream);
+  if (n_wide > 0 && n_wide_slots > 0) {
+    const int rc = launch_mfma_wide(a, dtype, n_wide_slots, stream);
     if (rc) return rc;
   }
   a.items += (long long)n_wide * VA_ITEM_WORDS;

@@ -1,7 +1,9 @@
 // Wide matrix-core view attention: query tiles of 128 (head_dim 256) or 256 MFMA rows, for
 // view-conditioned prefill (rows / G new tokens x G heads per workgroup).
 //
-// One workgroup of four waves per (work item, kv head), one wave per SIMD; wave w owns one
+// One workgroup of four waves per (slot, kv head), one wave per SIMD; a slot is one work item, or
+// several pieces of tiles whose walks add up to the same number of tokens in every slot, run one
+// after the other.  Wave w owns one
 // (head_dim 256) or two blocks of 32 MFMA rows (row R = tile row R / G, head R % G).  All waves walk
 // the same 32-token K/V tiles, which travel pool -> LDS directly (global_load_lds_dwordx4) into a
 // ring of four buffers: two tiles are in flight while the scores of a third and the products of a
@@ -103,13 +105,11 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   extern __shared__ va_u32x4 smem[];
   const char* lds = (const char*)smem;
 
+  // workgroup -> (slot, kv head); the slot's items are run one after the other
   const ItemHead where = item_and_head(blockIdx.x, a.num_kv_heads);
-  const int32_t* item = a.items + (long long)where.item * VA_ITEM_WORDS;
+  const int item_begin = a.wide_slots[where.item], item_end = a.wide_slots[where.item + 1];
   const int hk = where.head;
   const int G = a.num_q_heads / a.num_kv_heads;
-  const int n_q = item[VA_I_N_Q];
-  if (n_q == 0) return;  // padding item: keeps the launch order aligned with the die round-robin
-  const int part_base = item[VA_I_PART_BASE];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int lane = tid % kWave;
@@ -119,7 +119,6 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   int row_iq[kB];
 #pragma unroll
   for (int b = 0; b < kB; ++b) row_iq[b] = (row0 + 32 * b) / G;
-  const bool wave_active = (kWaveRows * wave) / G < n_q;  // the wave owns real rows
   const S* kp = (const S*)a.k_pool + (long long)hk * kD;
   const S* vp = (const S*)a.v_pool + (long long)hk * kD;
   const int P = a.page_size;
@@ -164,6 +163,13 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   const int v_base = v_row * kRowBytes + 16 * v_piece + 8 * (v_sub % 2);
   const int v_even = v_base + 64 * (v_swz >> 2), v_odd = v_base + 64 * (1 ^ (v_swz >> 2));
   const uint32_t lds_base = lds_address(lds);
+
+  for (int item_index = item_begin; item_index < item_end; ++item_index) {
+  const int32_t* item = a.items + (long long)item_index * VA_ITEM_WORDS;
+  const int n_q = item[VA_I_N_Q];
+  if (n_q == 0) continue;  // padding item
+  const int part_base = item[VA_I_PART_BASE];
+  const bool wave_active = (kWaveRows * wave) / G < n_q;  // the wave owns real rows
 
   float m_ref[kB], m_tile[kB], l_run[kB];  // reference maximum (log2 units), last tile maximum, row sum
   va_f32x16 o[kB][kDimTiles];
@@ -657,6 +663,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       }
     }
   }
+  }  // items of the slot
 }
 
 template <typename E, int kD>

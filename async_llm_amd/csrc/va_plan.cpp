@@ -31,6 +31,7 @@ namespace {
 struct Item {
   int32_t link_begin, n_links, n_q, part_base, tokens, kind;
   int32_t unit;  // items that stream the same K/V chunk share a unit (planner only, not serialised)
+  int32_t slot;  // wide items packed into one workgroup share a slot, -1: none (planner only)
 };
 constexpr int kXcds = 8;  // accelerator dies of an MI355X, each with its own L2; workgroup b runs on die b % 8
 struct Link {
@@ -44,6 +45,7 @@ struct Built {
   std::vector<int32_t> row_indptr;
   std::vector<int32_t> row_ids;
   std::vector<int32_t> row_flags;
+  std::vector<int32_t> wide_slots;  // indptr over the wide items: the items of each workgroup of the wide launch
   int32_t n_partials = 0;
   int32_t kernel = 0, q_tile = 0, kv_chunk = 0, wide_tile = 0, n_wide = 0;
 };
@@ -216,14 +218,16 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     cut_tiles((int64_t)gr.subrows.size(), tiles, wide_groups);
     total_tokens += (int64_t)tiles.size() * s->seq_lens[gr.rep];
   }
-  int64_t chain_tiles = 0, chain_tokens = 0;
+  int64_t chain_tiles = 0, chain_tokens = 0, wide_chain_tokens = 0;
   for (auto& ch : chains) {
     const int32_t nq = s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]];
     cut_tiles(nq, tiles);
     for (auto& tl : tiles) {
       ++chain_tiles;
-      for (int32_t m : ch)
-        chain_tokens += visible_end(s->seq_lens[m], nq, s->flags[m] & VA_SUB_CAUSAL, tl.second);
+      int64_t walked = 0;
+      for (int32_t m : ch) walked += std::max(0, visible_end(s->seq_lens[m], nq, s->flags[m] & VA_SUB_CAUSAL, tl.second));
+      chain_tokens += walked;
+      if (tl.second - tl.first > q_tile) wide_chain_tokens += walked;
     }
   }
   total_tokens += chain_tokens;
@@ -247,11 +251,12 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   std::vector<Pending> pend;
 
   int32_t next_unit = 0;
-  auto emit = [&](int32_t n_q, const std::vector<Link>& links, std::vector<int32_t>&& rows, int32_t unit = -1) {
+  auto emit = [&](int32_t n_q, const std::vector<Link>& links, std::vector<int32_t>&& rows, int32_t unit = -1,
+                  int32_t slot = -1) {
     int32_t tokens = 0;
     for (auto& l : links) tokens += l.tok_end - l.tok_begin;
     Item it{(int32_t)out.links.size(), (int32_t)links.size(), n_q, -1, tokens, n_q > q_tile ? 1 : 0,
-            unit >= 0 ? unit : next_unit++};
+            unit >= 0 ? unit : next_unit++, n_q > q_tile ? slot : -1};
     out.links.insert(out.links.end(), links.begin(), links.end());
     for (int32_t r : rows) ++row_count[r];
     pend.push_back(Pending{(int32_t)out.items.size(), std::move(rows)});
@@ -310,27 +315,61 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
         for (int32_t t0 = 0; t0 < len; t0 += per_w) emit_range(ti, t0, std::min(len, t0 + per_w));
   }
 
-  // Chains are split only when their tiles alone cannot fill the machine, and then by tokens: a
-  // tile gets one piece per `chain_budget` tokens it walks, so the tiles of a short request stay
-  // whole while those of a long one are cut (in a mixed batch the views differ by a factor of
-  // thirty; a uniform cut leaves the launch waiting for the longest).  The number of extra pieces
-  // over all tiles is at most chain_tokens / chain_budget <= want <= target.
+  // Chains.  When the tiles of all chains are many (several rounds of one workgroup per CU) every
+  // tile is one work item and the hardware hands them out as CUs fall free.  When they are few --
+  // a handful of prefill chunks in a continuous batch, whose views differ in length by a factor
+  // of thirty -- whole tiles cannot fill the machine evenly, so the walk of all tiles, laid end to
+  // end, is cut into equal token budgets instead: one budget per workgroup ("slot") of a launch of
+  // one workgroup per CU.  A slot runs its pieces one after the other; a tile cut in pieces yields
+  // partial states that the merge kernel folds.  Every slot then walks the same number of tokens
+  // (the cost of a wide tile is its tokens: all its rows share each K/V tile) and the launch is
+  // one even round, where 2.25 rounds of uneven items used to take the time of three.
+  // Narrow tiles of chains (the last rows of a request) are cut by the same budget, one item a piece.
+  const int64_t slots_wanted = std::max(1, 256 / shape->num_kv_heads);
   int64_t chain_budget = INT64_MAX;
-  if (chain_tiles > 0) {
-    // three rounds of work items over the CUs a head leaves to a launch of one workgroup per CU
-    const int64_t rounds = 3 * std::max(1, 256 / shape->num_kv_heads);
-    const int64_t want = std::max<int64_t>(1, std::min<int64_t>(target - (int64_t)out.items.size(), rounds));
-    // (a piece pays its own set-up -- the query tile is staged again -- so none is made for under ~1000 tokens)
-    if (chain_tiles < want) chain_budget = std::max<int64_t>((chain_tokens + want - 1) / want, 16 * gran);
+  // A piece stages its query tile again, which costs a wide tile about as much as walking this many
+  // tokens: the packing charges it to the slot's room, makes no piece shorter than it, and keeps a
+  // tile's remainder under it with the piece before.
+  const int32_t piece_cost = 6 * gran;
+  const int32_t min_piece = piece_cost;
+  if (chain_tiles > 0 && chain_tiles < 4 * slots_wanted) {
+    // (at most `want` <= target cuts are made, which is what bounds a fixed-capacity plan)
+    const int64_t want = std::max<int64_t>(1, std::min<int64_t>(target, slots_wanted));
+    const int64_t shared = wide_chain_tokens > 0 ? wide_chain_tokens : chain_tokens;
+    chain_budget = std::max<int64_t>((shared + want - 1) / want, 16 * gran);
   }
   // cuts inside a segment keep to multiples of 16 tokens where the kernels profit (pages of 16
   // tokens or more: a piece that starts on such a boundary is fetched with uniform loads)
   const bool align_cuts = shape->page_size >= 16 && (shape->page_size & (shape->page_size - 1)) == 0;
+  const bool pack = chain_budget != INT64_MAX;
+  // The room of a new wide slot is the even share of what is still to be placed over the slots
+  // still to be opened, so that a slot closed early (less than min_piece of its room left) or run
+  // over (a tile's short remainder kept with the piece before it) is made up for by the slots after
+  // it, and their number never exceeds the number wanted.
+  const int32_t slot_room = pack ? round_up(chain_budget + (align_cuts ? 15 : 0), gran) : 0;  // narrow tiles of chains
+  int64_t wide_tiles = 0;
+  for (auto& ch : chains) {
+    cut_tiles(s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]], tiles);
+    for (auto& tl : tiles) wide_tiles += tl.second - tl.first > q_tile;
+  }
+  int64_t slots_left = pack ? std::max<int64_t>(1, (wide_chain_tokens + chain_budget - 1) / chain_budget) : 0;
+  // what is still to be placed, set-ups included: a piece per slot or per tile, whichever are more,
+  // and another for about every other of those that are fewer (where a slot boundary falls inside a tile)
+  int64_t wide_left = wide_chain_tokens +
+                      piece_cost * (std::max(wide_tiles, slots_left) + std::min(wide_tiles, slots_left) / 2);
+  auto next_wide_room = [&]() -> int32_t {
+    if (slots_left <= 1) return INT32_MAX;  // the last slot takes whatever is left
+    const int64_t share = (wide_left + slots_left - 1) / slots_left;
+    --slots_left;
+    return round_up(share + (align_cuts ? 15 : 0), 16);
+  };
+  int32_t wide_slot = 0, wide_room = pack ? next_wide_room() : 0;  // the slot being filled with wide pieces
   for (auto& ch : chains) {
     const int32_t nq = s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]];
     cut_tiles(nq, tiles);
     for (auto& tl : tiles) {
       const int32_t a = tl.first, b = tl.second;
+      const bool wide = b - a > q_tile;
       std::vector<Link> all;
       int64_t tile_tokens = 0;
       for (int32_t m : ch) {
@@ -346,17 +385,40 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
       std::vector<int32_t> rows;
       for (int32_t r = a; r < b; ++r) rows.push_back((int32_t)s->sub_worker[s->qo_indptr[ch[0]] + r]);
       if (all.empty()) continue;
-      const int32_t parts = (int32_t)std::max<int64_t>(
-          1, std::min<int64_t>((tile_tokens + chain_budget / 2) / chain_budget, tile_tokens / (4 * gran)));
-      if (parts == 1) {
+      if (!pack) {
         emit(b - a, all, std::move(rows));
         continue;
       }
-      // an aligned cut may leave up to 15 tokens of a piece's room unused: the room allows for it, so
-      // that a tile never ends up in more than `parts` pieces
-      const int32_t per = round_up((tile_tokens + parts - 1) / parts + (align_cuts ? 15 : 0), gran);
+      // Cut the tile's walk where the room of the current budget ends.  Wide tiles fill the shared
+      // slots (the room carries over from tile to tile); a narrow tile starts a budget of its own.
+      int32_t room = wide ? wide_room : slot_room;
+      auto next_room = [&]() {
+        if (wide) ++wide_slot;
+        room = wide ? next_wide_room() : slot_room;
+      };
+      auto next_piece_room = [&]() {  // a further piece of this tile, in the next slot
+        next_room();
+        if (wide) {
+          room -= std::min(room, piece_cost);
+          wide_left -= piece_cost;
+        }
+      };
+      if (wide && room < piece_cost + min_piece) next_room();  // too little left for a piece worth its set-up
+      if (wide) {  // the set-up of the tile's first piece
+        room -= piece_cost;
+        wide_left -= piece_cost;
+      }
+      int64_t left = tile_tokens;  // tokens of the tile not yet in a piece
+      // no tiny last piece: a remainder under min_piece stays with the piece before it
+      auto fit_room = [&]() {
+        if (left > room && left - room < min_piece) room = (int32_t)left;
+      };
+      fit_room();
       std::vector<Link> cur;
-      int32_t room = per;
+      auto close_piece = [&]() {
+        if (!cur.empty()) emit(b - a, cur, std::vector<int32_t>(rows), -1, wide ? wide_slot : -1);
+        cur.clear();
+      };
       for (auto l : all) {
         const bool aligned = align_cuts && !(l.flags & VA_LINK_SLOTS);
         while (l.tok_begin < l.tok_end) {
@@ -364,9 +426,9 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
           if (aligned && take < l.tok_end - l.tok_begin) {
             take = take / 16 * 16;  // l.tok_begin is a multiple of 16: segments start at 0, cuts keep it so
             if (take == 0) {        // under 16 tokens of room left: the piece ends here
-              emit(b - a, cur, std::vector<int32_t>(rows));
-              cur.clear();
-              room = per;
+              close_piece();
+              next_piece_room();
+              fit_room();
               continue;
             }
           }
@@ -374,15 +436,21 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
           piece.tok_end = l.tok_begin + take;
           cur.push_back(piece);
           l.tok_begin += take;
+          left -= take;
           room -= take;
-          if (room == 0) {
-            emit(b - a, cur, std::vector<int32_t>(rows));
-            cur.clear();
-            room = per;
+          if (wide) wide_left -= take;
+          if (room <= 0 && left > 0) {
+            close_piece();
+            next_piece_room();
+            fit_room();
           }
         }
       }
-      if (!cur.empty()) emit(b - a, cur, std::vector<int32_t>(rows));
+      close_piece();
+      if (wide) {
+        if (room <= 0) next_room();
+        wide_room = room;
+      }
     }
   }
 
@@ -443,6 +511,33 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
       u.members.push_back(i);
     }
     if (units.empty()) continue;
+    if (kind == 1 && std::any_of(out.items.begin(), out.items.end(), [](const Item& it) { return it.kind == 1 && it.slot >= 0; })) {
+      // Packed wide pieces: every slot walks the same number of tokens, so the slots simply follow
+      // each other (slot k on die k % 8); wide items outside the packing get slots of their own.
+      std::vector<std::vector<int32_t>> by_slot;
+      for (int32_t i = 0; i < (int32_t)out.items.size(); ++i) {
+        const Item& it = out.items[i];
+        if (it.kind != 1) continue;
+        if (it.slot >= 0) {
+          if ((size_t)it.slot >= by_slot.size()) by_slot.resize(it.slot + 1);
+          by_slot[it.slot].push_back(i);
+        }
+      }
+      for (int32_t i = 0; i < (int32_t)out.items.size(); ++i)
+        if (out.items[i].kind == 1 && out.items[i].slot < 0) by_slot.push_back({i});
+      by_slot.erase(std::remove_if(by_slot.begin(), by_slot.end(), [](const std::vector<int32_t>& v) { return v.empty(); }),
+                    by_slot.end());
+      out.wide_slots.assign(1, 0);
+      for (auto& members : by_slot) {
+        for (int32_t m : members) sorted.push_back(out.items[m]);
+        out.wide_slots.push_back((int32_t)sorted.size());
+      }
+      while ((out.wide_slots.size() - 1) % kXcds) out.wide_slots.push_back((int32_t)sorted.size());  // empty slots
+      const Item padding{0, 0, 0, -1, 0, 1, -1, -1};
+      while (sorted.size() % kXcds) sorted.push_back(padding);  // outside every slot
+      out.n_wide = (int32_t)sorted.size();
+      continue;
+    }
     std::vector<int32_t> by_cost(units.size());
     std::iota(by_cost.begin(), by_cost.end(), 0);
     std::stable_sort(by_cost.begin(), by_cost.end(), [&](int32_t x, int32_t y) { return units[x].cost > units[y].cost; });
@@ -508,13 +603,18 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
         die_items[d].insert(die_items[d].end(), units[u].members.begin(), units[u].members.end());
       depth = std::max(depth, die_items[d].size());
     }
-    const Item padding{0, 0, 0, -1, 0, kind, -1};
+    const Item padding{0, 0, 0, -1, 0, kind, -1, -1};
     for (size_t slot = 0; slot < depth; ++slot)
       for (int d = 0; d < kXcds; ++d)
         sorted.push_back(slot < die_items[d].size() ? out.items[die_items[d][slot]] : padding);
-    if (kind == 1) out.n_wide = (int32_t)sorted.size();
+    if (kind == 1) {  // one workgroup per wide item
+      out.n_wide = (int32_t)sorted.size();
+      out.wide_slots.resize(out.n_wide + 1);
+      std::iota(out.wide_slots.begin(), out.wide_slots.end(), 0);
+    }
   }
   out.items.swap(sorted);
+  if (out.wide_slots.empty()) out.wide_slots.assign(1, 0);
   return VA_OK;
 }
 
@@ -529,8 +629,9 @@ void fill_counts(const Built& b, const VaSubRequests* s, const VaShape* shape, V
   c->n_qrefs = (int32_t)b.qrefs.size();
   c->n_partials = b.n_partials;
   c->n_row_parts = (int32_t)b.row_ids.size();
+  c->n_wide_slots = (int32_t)b.wide_slots.size() - 1;
   c->plan_words = VA_PLAN_HEADER_WORDS + c->n_items * VA_ITEM_WORDS + c->n_links * VA_LINK_WORDS +
-                  2 * c->n_qrefs + (s->n_rows + 1) + c->n_row_parts + s->n_rows;
+                  2 * c->n_qrefs + (s->n_rows + 1) + c->n_row_parts + s->n_rows + (c->n_wide_slots + 1);
   c->workspace_bytes = va_workspace_bytes_for(b.n_partials, shape->num_q_heads, shape->head_dim);
 }
 
@@ -572,6 +673,7 @@ static int write_plan(const Built& b, const VaSubRequests* subs, const VaShape* 
     cap_row_parts = cap->max_row_parts; cap_rows = cap->max_rows; cap_partials = cap->max_partials;
     c.n_items = cap_wide + cap_narrow;
     c.n_wide_items = cap_wide;
+    c.n_wide_slots = cap_wide;  // a fixed plan launches one workgroup per wide item it has room for
     c.n_links = cap_links;
     c.n_qrefs = cap_qrefs;
     c.n_partials = cap_partials;
@@ -623,9 +725,9 @@ static int write_plan(const Built& b, const VaSubRequests* subs, const VaShape* 
     }
   };
   for (int32_t i = 0; i < b.n_wide; ++i) write_item(i, b.items[i]);
-  for (int32_t i = b.n_wide; i < cap_wide; ++i) write_item(i, Item{0, 0, 0, -1, 0, 1, -1});
+  for (int32_t i = b.n_wide; i < cap_wide; ++i) write_item(i, Item{0, 0, 0, -1, 0, 1, -1, -1});
   for (int32_t i = 0; i < n_narrow; ++i) write_item(cap_wide + i, b.items[b.n_wide + i]);
-  for (int32_t i = n_narrow; i < cap_narrow; ++i) write_item(cap_wide + i, Item{0, 0, 0, -1, 0, 0, -1});
+  for (int32_t i = n_narrow; i < cap_narrow; ++i) write_item(cap_wide + i, Item{0, 0, 0, -1, 0, 0, -1, -1});
   off += (cap_wide + cap_narrow) * VA_ITEM_WORDS;
   h[VA_H_OFF_LINKS] = off;
   for (size_t i = 0; i < b.links.size(); ++i) {
@@ -656,6 +758,11 @@ static int write_plan(const Built& b, const VaSubRequests* subs, const VaShape* 
   std::copy(b.row_flags.begin(), b.row_flags.end(), plan_host + off);
   for (int32_t r = subs->n_rows; r < cap_rows; ++r) plan_host[off + r] = VA_ROW_EMPTY;
   off += cap_rows;
+  h[VA_H_N_WIDE_SLOTS] = c.n_wide_slots;
+  h[VA_H_OFF_WIDE_SLOTS] = off;
+  std::copy(b.wide_slots.begin(), b.wide_slots.end(), plan_host + off);
+  for (int32_t k = (int32_t)b.wide_slots.size(); k <= c.n_wide_slots; ++k) plan_host[off + k] = b.wide_slots.back();
+  off += c.n_wide_slots + 1;
   if (counts) *counts = c;
   return VA_OK;
 }
@@ -673,7 +780,7 @@ extern "C" int64_t va_plan_fixed_words(const VaPlanCapacity* cap) {
   if (!cap) return 0;
   return (int64_t)VA_PLAN_HEADER_WORDS + ((int64_t)cap->max_items + cap->max_wide_items) * VA_ITEM_WORDS +
          (int64_t)cap->max_links * VA_LINK_WORDS + 2 * (int64_t)cap->max_qrefs + (cap->max_rows + 1) +
-         cap->max_row_parts + cap->max_rows;
+         cap->max_row_parts + cap->max_rows + (cap->max_wide_items + 1);
 }
 
 // Upper bounds of every plan section for a workload within `lim`, following the rules of build():

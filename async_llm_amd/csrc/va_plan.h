@@ -36,6 +36,8 @@ enum {
   VA_H_N_WIDE,     // items [0, n_wide) are wide tiles, the rest narrow
   VA_H_WIDE_TILE,
   VA_H_OFF_QREF_ROWS,  // parallel to qrefs: the query/output row of each entry (sub_worker[qrefs[k]])
+  VA_H_N_WIDE_SLOTS,   // workgroups per kv head of the wide launch (a multiple of 8)
+  VA_H_OFF_WIDE_SLOTS, // [n_wide_slots + 1]: slot s runs the wide items [indptr[s], indptr[s + 1]) one after the other
 };
 
 // item word indices

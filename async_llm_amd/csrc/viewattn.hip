@@ -515,6 +515,8 @@ static int attention_launches(const void* q_dev, int64_t q_row_stride, const voi
   if (n_items % 8 || h[VA_H_N_WIDE] % 8 || h[VA_H_N_WIDE] < 0 || h[VA_H_N_WIDE] > n_items)
     return va_fail(VA_ERR_ARG, "plan header: item counts (%d, %d wide) are not padded to the 8 dies", n_items,
                    h[VA_H_N_WIDE]);
+  if (h[VA_H_N_WIDE_SLOTS] % 8 || h[VA_H_N_WIDE_SLOTS] < 0 || h[VA_H_N_WIDE_SLOTS] > h[VA_H_N_WIDE])
+    return va_fail(VA_ERR_ARG, "plan header: %d wide slots for %d wide items", h[VA_H_N_WIDE_SLOTS], h[VA_H_N_WIDE]);
   if (!out_dev) return va_fail(VA_ERR_ARG, "null out");
   if (n_items > 0 && (!q_dev || !k_pool_dev || !v_pool_dev || !sub_worker_dev || !sub_loc_dev || !kv_indices_dev))
     return va_fail(VA_ERR_ARG, "null pointer");
@@ -537,6 +539,7 @@ static int attention_launches(const void* q_dev, int64_t q_row_stride, const voi
   a.links = plan_dev + h[VA_H_OFF_LINKS];
   a.qrefs = plan_dev + h[VA_H_OFF_QREFS];
   a.qref_rows = plan_dev + h[VA_H_OFF_QREF_ROWS];
+  a.wide_slots = plan_dev + h[VA_H_OFF_WIDE_SLOTS];
   a.kv_indices = kv_indices_dev;
   a.sub_worker = sub_worker_dev;
   a.sub_loc = sub_loc_dev;
@@ -556,7 +559,7 @@ static int attention_launches(const void* q_dev, int64_t q_row_stride, const voi
 
   if (n_items > 0) {
     if (h[VA_H_KERNEL] == VA_KERNEL_MFMA) {
-      rc = va::launch_mfma(a, shape->dtype, n_items, h[VA_H_N_WIDE], h[VA_H_Q_TILE], s);
+      rc = va::launch_mfma(a, shape->dtype, n_items, h[VA_H_N_WIDE], h[VA_H_N_WIDE_SLOTS], h[VA_H_Q_TILE], s);
     } else {
       VA_DISPATCH_DTYPE(shape->dtype, rc = va::launch_generic<E>(a, n_items, s));
     }

@@ -103,6 +103,7 @@ class VaPlanCounts(C.Structure):
         ("wide_tile", C.c_int32),
         ("n_wide_items", C.c_int32),
         ("workspace_bytes", C.c_int64),
+        ("n_wide_slots", C.c_int32),
     ]
 
 

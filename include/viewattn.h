@@ -163,6 +163,8 @@ typedef struct VaPlanCounts {
   int32_t wide_tile;     /* resolved rows of a wide tile (0: none)           */
   int32_t n_wide_items;  /* items served by the wide kernel                  */
   int64_t workspace_bytes; /* device scratch va_attention needs for this plan */
+  int32_t n_wide_slots;  /* workgroups per kv head of the wide launch (a multiple of 8): a slot
+                            runs one wide item, or several pieces of equal total length */
 } VaPlanCounts;
 
 /* Size the plan (no output besides *counts). */
@@ -175,7 +177,7 @@ VA_API int va_plan_count(const VaSubRequests* subs, const VaShape* shape, const 
  * device verbatim and pass the device copy to va_attention.  Layout (int32
  * words): header[24] | items[n_items*16] | links[n_links*8] | qrefs[n_qrefs] |
  * qref_rows[n_qrefs] | row_part_indptr[n_rows+1] | row_part_ids[n_row_parts] |
- * row_flags[n_rows].  (An item carries a copy of its first link, and qref_rows
+ * row_flags[n_rows] | wide_slots[n_wide_slots+1].  (An item carries a copy of its first link, and qref_rows
  * the output row of every qrefs entry: both shorten the chain of dependent loads
  * at the start of a workgroup.)
  * Items are in launch order, laid out for the 8 dies of an MI355X (workgroup b

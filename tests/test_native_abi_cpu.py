@@ -15,7 +15,7 @@ from async_llm_amd import native
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 H = dict(MAGIC=0, KERNEL=1, Q_TILE=2, KV_CHUNK=3, N_ITEMS=4, N_LINKS=5, N_QREFS=6, N_PARTIALS=7, N_ROW_PARTS=8,
          N_ROWS=9, OFF_ITEMS=10, OFF_LINKS=11, OFF_QREFS=12, OFF_ROW_INDPTR=13, OFF_ROW_IDS=14, OFF_ROW_FLAGS=15,
-         N_EMPTY=16, N_SUBROWS=17, N_WIDE=18, WIDE_TILE=19, OFF_QREF_ROWS=20)
+         N_EMPTY=16, N_SUBROWS=17, N_WIDE=18, WIDE_TILE=19, OFF_QREF_ROWS=20, N_WIDE_SLOTS=21, OFF_WIDE_SLOTS=22)
 NO_CAUSAL = 0x3FFFFFFF
 
 
@@ -78,6 +78,10 @@ def check_coverage(blob, qo, kvp, lens, flags, sub_worker, n_rows, fixed=False):
     # each class (wide first, then narrow) is padded to a multiple of the 8 dies
     assert h[H["N_WIDE"]] % 8 == 0 and h[H["N_ITEMS"]] % 8 == 0
     assert all(it[5] == 1 for it in items[: h[H["N_WIDE"]]]) and all(it[5] == 0 for it in items[h[H["N_WIDE"]]:])
+    # the wide launch runs one workgroup per slot: the slots partition the real wide items, in order
+    slots = blob[h[H["OFF_WIDE_SLOTS"]]: h[H["OFF_WIDE_SLOTS"]] + h[H["N_WIDE_SLOTS"]] + 1]
+    assert h[H["N_WIDE_SLOTS"]] % 8 == 0 and slots[0] == 0 and all(a <= b for a, b in zip(slots, slots[1:]))
+    assert slots[-1] <= h[H["N_WIDE"]] and all(it[2] == 0 for it in items[slots[-1]: h[H["N_WIDE"]]])
     for it in items:
         lb, nl, nq, part_base = it[0], it[1], it[2], it[3]
         if nq == 0:  # padding item
@@ -309,6 +313,42 @@ def test_compute_entry_points_refuse_cpu_tensors():
 
     with pytest.raises(native.ViewAttnError, match="GPU only"):
         apply_rope_correction(torch.zeros(2, 1, 8), torch.zeros(2, dtype=torch.int64), torch.zeros(4, 8))
+
+
+def test_few_wide_tiles_are_packed_into_slots_of_equal_length():
+    """Four prefill chunks of 64 tokens (two wide tiles each at 16 q / 4 kv heads of 256 dims) over
+    views of 1.5k to 30k tokens: 8 tiles cannot fill 64 workgroup slots per kv head, and cut one
+    by one into similar pieces they would still fill them unevenly.  The planner lays all walks
+    end to end and gives every slot the same share; a slot holds the end of one tile and the start
+    of the next."""
+    page = 16
+    qo, kvp, kvi, lens, flags, chain, sw = [0], [0], [], [], [], [], []
+    n_rows = 0
+    for r, context in enumerate((30000, 1500, 12345, 22222)):
+        rows = list(range(n_rows, n_rows + 64))
+        n_rows += 64
+        for L in (512, context):
+            kvi += list(range(len(kvi), len(kvi) + -(-L // page)))
+            kvp.append(len(kvi)); lens.append(L); flags.append(0); chain.append(r)
+            sw += rows; qo.append(len(sw))
+        kvi += list(range(len(kvi), len(kvi) + -(-(100 + 64) // page)))
+        kvp.append(len(kvi)); lens.append(164); flags.append(1); chain.append(r)
+        sw += rows; qo.append(len(sw))
+    rc, blob, counts = build_plan(qo, kvp, kvi, lens, flags, chain, sw, n_rows, heads=(16, 4, 256), page=page,
+                                  dtype=native.VA_BF16, kernel=native.VA_KERNEL_MFMA)
+    assert rc == 0
+    check_coverage(blob, qo, kvp, lens, flags, sw, n_rows)
+    h, items, links, *_ = decode_plan(blob)
+    slots = blob[h[H["OFF_WIDE_SLOTS"]]: h[H["OFF_WIDE_SLOTS"]] + h[H["N_WIDE_SLOTS"]] + 1]
+    assert counts.n_wide_slots == h[H["N_WIDE_SLOTS"]] == 64 and counts.n_wide_items >= 64
+    total = 2 * (4 * 512 + 30000 + 1500 + 12345 + 22222) + sum(2 * 100 + 32 + 64 for _ in range(4))
+    assert int(items[: slots[-1], 4].sum()) == total
+    # a slot's load: the tokens it walks plus the set-up of each of its pieces (worth ~384 tokens)
+    load = [int(items[a:b, 4].sum()) + 384 * int(b - a) for a, b in zip(slots, slots[1:])]
+    mean = sum(load) / 64
+    # the longest slot sets the time of the launch (the last slot takes what is left and may be short)
+    assert max(load) <= 1.06 * mean and min(load) > 0 and sorted(load)[1] >= 0.9 * mean, (min(load), max(load), mean)
+    assert min(int(it[4]) for it in items[: slots[-1]]) >= 384 - 16  # no piece too short to be worth its set-up
 
 
 def test_prefill_tiles_are_cut_by_tokens_on_page_group_boundaries():
