@@ -54,8 +54,8 @@ def _compile_one(hipcc, src, obj, extra, verbose):
              verbose)
         _run([hipcc, *COMMON_FLAGS, *HOST_FLAGS, *extra, "-Xclang", "-fcuda-include-gpubinary", "-Xclang", fatbin,
               "-c", path, "-o", obj], verbose)
-    else:
-        _run([hipcc, *COMMON_FLAGS, *extra, "-c", path, "-o", obj], verbose)
+    else:  # host code only (hipcc would take a .cpp for HIP and run a device pass over it)
+        _run([os.environ.get("CXX", "g++"), *COMMON_FLAGS, *extra, "-c", path, "-o", obj], verbose)
 
 
 def build(verbose: bool = True, out: str = LIB_PATH, extra_flags=(), incremental: bool = False) -> str:

@@ -116,14 +116,94 @@ __global__ __launch_bounds__(256) void rope_store_kernel(
   }
 }
 
+// The same in 16-byte pieces, for rows whose addresses, strides and rotary half are multiples of
+// a piece (the reference's store kernel copies with 16-byte vectors too: store.cu:42-54).  Thread j
+// of a row takes key unit j -- a rotary pair of pieces (dims [i0, i0 + kVec) and the same dims half
+// a rotary_dim further: one thread reads both, rotates element by element with the arithmetic of
+// rope_pair, writes both, so in place is safe) or a piece past the rotary part -- and value piece j;
+// all of a thread's loads are issued before its first store.  Consecutive threads take consecutive
+// pieces of consecutive rows: a workgroup covers one row or several, whatever the row length.
+template <typename E>
+__global__ __launch_bounds__(256) void rope_store_vec_kernel(
+    const typename E::storage* __restrict__ x, const typename E::storage* __restrict__ v,
+    typename E::storage* y, typename E::storage* v_out, long long x_stride, long long v_stride,
+    long long y_stride, const void* dst, int dst_is_i64, const int64_t* pos, long long pos_axis_stride,
+    long long n_rows, int n_heads, int head_dim, RopeDev rope, int pair_units, int key_units, int units) {
+  using S = typename E::storage;
+  constexpr int kVec = 16 / sizeof(S);
+  union Piece {
+    uint4 raw;
+    S e[kVec];
+  };
+  const unsigned idx = blockIdx.x * 256u + threadIdx.x;  // the launcher keeps rows * units within 32 bits
+  const long long row = idx / (unsigned)units;
+  if (row >= n_rows) return;
+  const int u = (int)(idx - (unsigned)row * (unsigned)units);
+  long long out_row = row;
+  if (dst) {
+    out_row = dst_is_i64 ? ((const long long*)dst)[row] : (long long)((const int*)dst)[row];
+    if (out_row < 0) return;
+  }
+  const S* xr = x + row * x_stride;
+  S* yr = y + out_row * y_stride;
+  const bool has_value = v != nullptr && u < n_heads * (head_dim / kVec);
+  Piece val, xa, xb, ya, yb;
+  if (has_value) val.raw = *(const uint4*)(v + row * v_stride + u * kVec);
+  int ea = -1, eb = -1;  // element offsets of the key pieces this thread writes
+  if (u < pair_units) {
+    const int per_head = rope.half / kVec;
+    const int h = u / per_head, i0 = (u - h * per_head) * kVec;
+    ea = h * head_dim + i0;
+    eb = ea + rope.half;
+    xa.raw = *(const uint4*)(xr + ea);
+    xb.raw = *(const uint4*)(xr + eb);
+    const Pos3 p = load_pos(pos, pos_axis_stride, row);
+#pragma unroll
+    for (int k = 0; k < kVec; ++k) {
+      float c, sn, y1, y2;
+      rope_cos_sin(rope, p, i0 + k, c, sn);
+      rope_pair<E>(rope, c, sn, E::load(xa.e[k]), E::load(xb.e[k]), y1, y2);
+      ya.e[k] = E::store(y1);
+      yb.e[k] = E::store(y2);
+    }
+  } else if (u < key_units) {  // a key piece past the rotary part
+    const int t = u - pair_units, per_head = (head_dim - rope.rotary_dim) / kVec;
+    ea = (t / per_head) * head_dim + rope.rotary_dim + (t % per_head) * kVec;
+    ya.raw = *(const uint4*)(xr + ea);
+  }
+  if (has_value) *(uint4*)(v_out + out_row * y_stride + u * kVec) = val.raw;
+  if (ea >= 0) *(uint4*)(yr + ea) = ya.raw;
+  if (eb >= 0) *(uint4*)(yr + eb) = yb.raw;
+}
+
 template <typename E>
 int launch_rope_store(const void* x, const void* v, void* y, void* v_out, long long x_stride,
                       long long v_stride, long long y_stride, const void* dst, int dst_is_i64,
                       const int64_t* pos, long long pos_axis_stride, long long n_rows, int n_heads,
                       int head_dim, const RopeDev& rope, hipStream_t stream) {
   using S = typename E::storage;
+  constexpr int kVec = 16 / sizeof(S);
   if (n_rows == 0) return VA_OK;
   if (n_rows > 0x7fffffffLL) return va_fail(VA_ERR_ARG, "too many rows");
+  auto piecewise = [&](const void* ptr, long long stride) {
+    return ptr == nullptr || ((uintptr_t)ptr % 16 == 0 && stride % kVec == 0);
+  };
+  const bool vec = head_dim % kVec == 0 && rope.half % kVec == 0 && piecewise(x, x_stride) && piecewise(y, y_stride) &&
+                   piecewise(v, v_stride) && piecewise(v_out, y_stride);
+  if (vec) {
+    const bool copy_tail = x != y || dst != nullptr;
+    const int pair_units = n_heads * (rope.half / kVec);
+    const int key_units = pair_units + (copy_tail ? n_heads * ((head_dim - rope.rotary_dim) / kVec) : 0);
+    const int units = v ? n_heads * (head_dim / kVec) : key_units;  // (key_units <= the pieces of a row)
+    if (units > 0 && n_rows * units < 0x7fffff00LL) {
+      const long long blocks = (n_rows * units + 255) / 256;
+      hipLaunchKernelGGL(rope_store_vec_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, stream, (const S*)x,
+                         (const S*)v, (S*)y, (S*)v_out, x_stride, v_stride, y_stride, dst, dst_is_i64, pos,
+                         pos_axis_stride, n_rows, n_heads, head_dim, rope, pair_units, key_units, units);
+      return check_hip(hipGetLastError(), "rope/store launch");
+    }
+    if (units == 0) return VA_OK;
+  }
   hipLaunchKernelGGL(rope_store_kernel<E>, dim3((unsigned)n_rows), dim3(256), 0, stream, (const S*)x,
                      (const S*)v, (S*)y, (S*)v_out, x_stride, v_stride, y_stride, dst, dst_is_i64, pos,
                      pos_axis_stride, n_rows, n_heads, head_dim, rope);
