@@ -292,50 +292,80 @@ class SharedCacheAttention:
 
     def _walk_decode(self, group, new_page_for_block, new_token_slots):
         """Sub-requests of one decode step: per worker one paged sub-request per
-        non-empty view block, plus a single-slot one when it writes outside its view."""
+        non-empty view block, plus a single-slot one when it writes outside its
+        view (reference ``attention.py:326-370``).  The (worker, block) pairs are
+        walked once to number the distinct blocks; lengths, spans, rotation
+        offsets and segment slots are then array arithmetic over those numbers.
+        Returns ``main`` / ``aux`` tables (int64 arrays, ``pages`` a list of int32
+        arrays) in the reference's order, and the largest segment count."""
         W = group.num_workers
         assert W > 0
         P = self.page_size
-        written = set(new_page_for_block)
-        snapshot: Dict[int, np.ndarray] = {}
         views, targets = group.cache_structure, group.write_to
 
-        main = {"worker": [], "loc": [], "slot": [], "pages": [], "n_pages": [], "len": [], "last": []}
-        aux = {"worker": [], "loc": [], "slot": [], "kv": []}
-        slots_host: Optional[list] = None
-        max_segments = 0
+        number: Dict[int, int] = {}  # id(block) -> index into `blocks`
+        blocks: list = []
+        flat: List[int] = []  # block number of every (worker, view position), worker-major
+        counts = np.empty(W, dtype=np.int64)
+        for w, view in enumerate(views):
+            counts[w] = len(view)
+            for b in view:
+                k = number.get(id(b))
+                if k is None:
+                    k = number[id(b)] = len(blocks)
+                    blocks.append(b)
+                flat.append(k)
+        n_blocks = len(blocks)
+        tokens = np.fromiter((b.num_tokens for b in blocks), dtype=np.int64, count=n_blocks)
+        spans = np.fromiter((b.mrope_span for b in blocks), dtype=np.int64, count=n_blocks)
+        grow = np.fromiter((id(b) in new_page_for_block for b in blocks), dtype=np.int64, count=n_blocks)
+        tokens += grow  # this step's appends are stored before any attention runs
+        spans += grow
 
-        for w in range(W):
-            view, target = views[w], targets[w]
-            grow = [1 if id(b) in written else 0 for b in view]
-            total_span = sum(b.mrope_span + g for b, g in zip(view, grow))
-            before = 0  # span of the blocks ahead of the current one
-            seg = 0
-            for b, g in zip(view, grow):
-                length = b.num_tokens + g
-                if length:
-                    pages = page_numbers_array(b, snapshot, new_page_for_block.get(id(b)))
-                    main["worker"].append(w)
-                    main["loc"].append(total_span - before - 1)
-                    main["slot"].append(seg)
-                    main["pages"].append(pages)
-                    main["n_pages"].append(len(pages))
-                    main["len"].append(length)
-                    main["last"].append(length - (len(pages) - 1) * P)
-                    seg += 1
-                before += b.mrope_span + g
-            if not any(b is target for b in view):
-                # the writer still attends to the token it writes, at distance 0
-                if slots_host is None:
-                    slots_host = new_token_slots.cpu().tolist()
-                aux["worker"].append(w)
-                aux["loc"].append(target.mrope_span)
-                aux["slot"].append(seg)
-                aux["kv"].append(slots_host[w])
-                seg += 1
-            max_segments = max(max_segments, seg)
+        flat_arr = np.asarray(flat, dtype=np.int64)
+        worker = np.repeat(np.arange(W, dtype=np.int64), counts)
+        first = np.concatenate(([0], np.cumsum(counts)[:-1]))  # first pair of each worker
+        span = spans[flat_arr]
+        length = tokens[flat_arr]
+        ahead = np.cumsum(span) - span  # span of all pairs before this one ...
+        total = np.bincount(worker, weights=span, minlength=W).astype(np.int64)  # exact: spans are far below 2^53
+        base = np.zeros(W, dtype=np.int64)
+        has_view = counts > 0
+        base[has_view] = ahead[first[has_view]]
+        ahead -= base[worker]  # ... and of the blocks ahead of it in its own view
+        live = length > 0
+        seen = np.cumsum(live) - live
+        seg_base = np.zeros(W, dtype=np.int64)
+        seg_base[has_view] = seen[first[has_view]]
+        segments = np.bincount(worker[live], minlength=W)
 
-        return main, aux, max_segments
+        snapshot: Dict[int, np.ndarray] = {}
+        page_of_block: List[Optional[np.ndarray]] = [None] * n_blocks
+        pages = []
+        for k in flat_arr[live].tolist():
+            got = page_of_block[k]
+            if got is None:
+                b = blocks[k]
+                got = page_of_block[k] = page_numbers_array(b, snapshot, new_page_for_block.get(id(b)))
+            pages.append(got)
+        n_pages = np.fromiter((len(p) for p in pages), dtype=np.int64, count=len(pages))
+        main = {"worker": worker[live], "loc": (total[worker] - ahead - 1)[live], "slot": (seen - seg_base[worker])[live],
+                "pages": pages, "n_pages": n_pages, "len": length[live]}
+        main["last"] = main["len"] - (n_pages - 1) * P
+
+        # a writer whose block is outside its view still attends to the token it writes, at distance 0
+        target_no = np.fromiter((number.get(id(t), -1) for t in targets), dtype=np.int64, count=W)
+        inside = np.zeros(W, dtype=bool)
+        inside[worker[flat_arr == target_no[worker]]] = True
+        outside = np.nonzero(~inside)[0]
+        aux = {"worker": outside, "loc": np.fromiter((targets[w].mrope_span for w in outside.tolist()), dtype=np.int64,
+                                                      count=len(outside)),
+               "slot": segments[outside], "kv": np.zeros(0, dtype=np.int64)}
+        if len(outside):
+            aux["kv"] = new_token_slots.cpu().numpy().astype(np.int64)[outside]
+            segments = segments.copy()
+            segments[outside] += 1
+        return main, aux, int(segments.max())
 
     def prepare(
         self,
@@ -366,30 +396,31 @@ class SharedCacheAttention:
             parts.append(aux["kv"])
         kv_indices = upload_page_indices(parts, self.device, refs)
         kv_host = refs[0]
-        n_main_entries = sum(main["n_pages"])
+        n_main_entries = int(main["n_pages"].sum())
+        main_indptr = np.concatenate(([0], np.cumsum(main["n_pages"])))
 
         main_plan = aux_plan = None
         if n_main:
-            main_plan = dict(indptr=_cumulative(main["n_pages"]), indices=kv_host[:n_main_entries],
-                             last_page_len=_i32(main["last"]), seq_lens=_i32(main["len"]), page_size=P)
+            main_plan = dict(indptr=torch.from_numpy(main_indptr.astype(np.int32)), indices=kv_host[:n_main_entries],
+                             last_page_len=torch.from_numpy(main["last"].astype(np.int32)),
+                             seq_lens=torch.from_numpy(main["len"].astype(np.int32)), page_size=P)
         if n_aux:
             aux_plan = dict(indptr=torch.arange(n_aux + 1, dtype=torch.int32), indices=kv_host[n_main_entries:],
                             last_page_len=torch.ones(n_aux, dtype=torch.int32),
                             seq_lens=torch.ones(n_aux, dtype=torch.int32), page_size=1)
 
-        sub_worker = main["worker"] + aux["worker"]
-        sub_loc = main["loc"] + aux["loc"]
-        sub_slot = main["slot"] + aux["slot"]
-        pad_slot = [w * max_segments + s for w, s in zip(sub_worker, sub_slot)]
+        sub_worker = np.concatenate([main["worker"], aux["worker"]])
+        sub_loc = np.concatenate([main["loc"], aux["loc"]])
+        pad_slot = sub_worker * max_segments + np.concatenate([main["slot"], aux["slot"]])
         n_sub = n_main + n_aux
 
         launch = self._build_launch(
             qo_indptr=np.arange(n_sub + 1),
-            kv_indptr=np.concatenate([np.cumsum([0] + main["n_pages"]), n_main_entries + 1 + np.arange(n_aux)]),
+            kv_indptr=np.concatenate([main_indptr, n_main_entries + 1 + np.arange(n_aux)]),
             kv_indices_host=kv_host.numpy(),
-            seq_lens=main["len"] + [1] * n_aux,
-            flags=[0] * n_main + [native.VA_SUB_SLOTS] * n_aux,
-            chain=[-1] * n_sub,
+            seq_lens=np.concatenate([main["len"], np.ones(n_aux, dtype=np.int64)]),
+            flags=np.concatenate([np.zeros(n_main, dtype=np.int32), np.full(n_aux, native.VA_SUB_SLOTS, dtype=np.int32)]),
+            chain=np.full(n_sub, -1, dtype=np.int32),
             sub_worker_host=sub_worker,
             n_rows=W, kv_indices_dev=kv_indices, refs=refs)
 
@@ -404,7 +435,7 @@ class SharedCacheAttention:
     def _upload_i64(self, rows: Sequence, refs: list) -> List[torch.Tensor]:
         """One pinned staging tensor and one async copy for several equally long
         int64 tables; returns the device rows."""
-        host = torch.tensor(rows, dtype=torch.int64).reshape(len(rows), -1)
+        host = torch.from_numpy(np.stack([np.asarray(r, dtype=np.int64) for r in rows]))
         if self.device.type == "cuda":
             host = host.pin_memory()
         dev = host.to(self.device, non_blocking=True)
@@ -552,11 +583,11 @@ class SharedCacheAttention:
         parts = list(main["pages"]) + ([aux["kv"]] if n_aux else []) + ctx["pages"] + own["pages"]
         kv_indices = upload_page_indices(parts, self.device, refs)
         kv_host = refs[0]
-        kv_counts = main["n_pages"] + [1] * n_aux + ctx["n_pages"] + own["n_pages"]
+        kv_counts = main["n_pages"].tolist() + [1] * n_aux + ctx["n_pages"] + own["n_pages"]
 
-        dec_worker = np.asarray(main["worker"] + aux["worker"], dtype=np.int64)
-        dec_slot = np.asarray(main["slot"] + aux["slot"], dtype=np.int64)
-        dec_loc = torch.tensor(main["loc"] + aux["loc"], dtype=torch.int64)
+        dec_worker = np.concatenate([main["worker"], aux["worker"]])
+        dec_slot = np.concatenate([main["slot"], aux["slot"]])
+        dec_loc = torch.from_numpy(np.concatenate([main["loc"], aux["loc"]]))
         pre_rows = np.concatenate(ctx["rows"] + own["rows"]) + W
         pre_slot = np.concatenate(ctx["slot"] + own["slot"])
         pre_loc = torch.cat(ctx["loc"] + own["loc"], dim=1 if use_3d else 0)
@@ -570,7 +601,7 @@ class SharedCacheAttention:
             qo_indptr=np.cumsum([0] + [1] * (n_main + n_aux) + ctx["q"] + own["q"]),
             kv_indptr=np.cumsum([0] + kv_counts),
             kv_indices_host=kv_host.numpy(),
-            seq_lens=main["len"] + [1] * n_aux + ctx["len"] + own["len"],
+            seq_lens=main["len"].tolist() + [1] * n_aux + ctx["len"] + own["len"],
             flags=[0] * n_main + [native.VA_SUB_SLOTS] * n_aux + [0] * n_ctx + [native.VA_SUB_CAUSAL] * n_self,
             chain=[-1] * (n_main + n_aux) + ctx["chain"] + own["chain"],
             sub_worker_host=sub_worker,
