@@ -527,12 +527,18 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
         if (out.items[i].kind == 1 && out.items[i].slot < 0) by_slot.push_back({i});
       by_slot.erase(std::remove_if(by_slot.begin(), by_slot.end(), [](const std::vector<int32_t>& v) { return v.empty(); }),
                     by_slot.end());
+      // Slots were filled in the order of the tiles, so neighbouring slots walk the same request's
+      // view (the pieces of one chunk's query tiles) at the same pace: they go to ONE die, where the
+      // K/V they share is fetched from HBM once and found in that die's L2 by the others.  Slot k of
+      // the launch runs on die k % 8: die d takes the d-th run of n / 8 consecutive slots.
+      while (by_slot.size() % kXcds) by_slot.emplace_back();  // empty slots
+      const size_t per_die = by_slot.size() / kXcds;
       out.wide_slots.assign(1, 0);
-      for (auto& members : by_slot) {
+      for (size_t k = 0; k < by_slot.size(); ++k) {
+        const auto& members = by_slot[(k % kXcds) * per_die + k / kXcds];
         for (int32_t m : members) sorted.push_back(out.items[m]);
         out.wide_slots.push_back((int32_t)sorted.size());
       }
-      while ((out.wide_slots.size() - 1) % kXcds) out.wide_slots.push_back((int32_t)sorted.size());  // empty slots
       const Item padding{0, 0, 0, -1, 0, 1, -1, -1};
       while (sorted.size() % kXcds) sorted.push_back(padding);  // outside every slot
       out.n_wide = (int32_t)sorted.size();

@@ -385,7 +385,7 @@ def test_prefill_tiles_are_cut_by_tokens_on_page_group_boundaries():
             weight.setdefault(long_one, []).append(tokens)
         assert len(weight[False]) == 1, "the short tile was cut"
         assert len(weight[True]) >= 20, "the long tile was not cut by its tokens"
-        assert max(weight[True]) <= 1.3 * min(w for w in weight[True][:-1]), weight[True]
+        assert max(weight[True]) <= 1.3 * sorted(weight[True])[1], weight[True]  # (one piece takes what is left)
         inner = [int(l[1]) for it in real for l in links[it[0]: it[0] + it[1]] if l[1] > 0]
         assert inner, "no cut inside a segment"
         if page >= 16:
