@@ -126,30 +126,42 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   const int p_shift = __builtin_ctz(P);  // t / P and t % P as shift and mask (power-of-two pages)
   const int row_bytes = (int)a.pool_row_stride * (int)sizeof(S);
 
-  // this lane's part of a wave-level load: row within the load and (swizzled) piece; waves 0 and 1
-  // load K halves, waves 2 and 3 V halves, each kind with its own swizzle
+  // This lane's part of a wave-level load (64 lanes x 16 bytes land as one 1 KB run in LDS; which
+  // piece of the pool a lane fetches is free).  Waves 0 and 1 load K halves, waves 2 and 3 V halves.
+  //   V: load u covers kRowsPerLoad whole rows, piece c of row r at position c ^ vswz(r).
+  //   K: fragment order.  Load u of a half is the block (8 rows R, 128-byte column g) = the operands
+  //      of four contraction steps for eight tokens: lane 16 s2 + 8 (h ^ R % 2) + j3 fetches row
+  //      8 R + j3, piece 8 g + 2 s2 + h.  The block of step s = 4 g + s2 thus lies 256 s bytes into
+  //      the 8-row region of R, and the fragment reads of a tile are ONE per-lane address plus
+  //      immediates; 16 consecutive lanes (served together) read 256 consecutive bytes, the flip of
+  //      h in odd R keeps the two regions they straddle on different banks.
   const bool wave_is_v = wave >= 2;
-  auto ld_swz = [&](int r) __attribute__((always_inline)) { return wave_is_v ? wide_vswz(r) : wide_swz<kD>(r); };
+  constexpr int kColumns = kChunks / 8;  // 128-byte columns of a row
   const int ld_row0 = lane / kChunks;
-  const int ld_x0 = (lane % kChunks) ^ ld_swz(ld_row0);
-  // byte offset, from the first row of its 16-token group, of what this lane fetches in load u of a
-  // tile that lies entirely inside the visible range (uniform pages)
+  const int ld_x0 = (lane % kChunks) ^ wide_vswz(ld_row0);
+  auto ld_row = [&](int u) __attribute__((always_inline)) {  // row within the wave's 16-token half
+    return wave_is_v ? u * Sh::kRowsPerLoad + ld_row0 : 8 * (u / kColumns) + lane % 8;
+  };
+  auto ld_piece = [&](int u) __attribute__((always_inline)) {
+    return wave_is_v ? (ld_x0 ^ wide_vswz(u * Sh::kRowsPerLoad))
+                     : 8 * (u % kColumns) + 2 * (lane / 16) + (((lane / 8) ^ (u / kColumns)) & 1);
+  };
+  // The loads of a plain tile (uniform pages, inside the visible range) go out in groups of up to four
+  // behind one setting of M0, as a wave-uniform base plus a per-lane offset that never changes.  A
+  // group's immediate offsets move the pool address as well: the per-lane offsets have them taken
+  // off beforehand (grouped_lane_offset) and carry a bias, which the base gives back, to stay positive.
+  constexpr int kLoadBias = 3072;
   uint32_t ld_off[kL];
 #pragma unroll
   for (int u = 0; u < kL; ++u)
-    ld_off[u] = grouped_lane_offset(
-        (uint32_t)((u * Sh::kRowsPerLoad + ld_row0) * row_bytes + 16 * (ld_x0 ^ ld_swz(u * Sh::kRowsPerLoad))), u);
-  // the loads of a plain tile go out in groups of up to four behind one setting of M0; a group's
-  // rows start at least 1024 bytes apart in the pool (kRowsPerLoad rows of at least 2 D bytes), so
-  // the offsets stay non-negative after the adjustment
+    ld_off[u] = grouped_lane_offset((uint32_t)(ld_row(u) * row_bytes + 16 * ld_piece(u) + kLoadBias), u);
   constexpr int kLoadGroup = kL >= 4 ? 4 : kL;
   auto issue_plain = [&](const char* base, uint32_t dst) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < kL; u += kLoadGroup) load_group_to_lds<kLoadGroup>(base, ld_off + u, dst + u * 1024);
   };
   // LDS offsets of what this lane reads from a tile
-  const int swz_j = wide_swz<kD>(j);
-  const int k_row_byte = j * kRowBytes;
+  const int k_lane_byte = (j / 8) * 8 * kRowBytes + 128 * ((h ^ (j / 8)) & 1) + 16 * (j % 8);
   // V^T fragments come from transposing reads.  For dim tile t (dims 32t .. 32t+31) and 16-token
   // step kk the lane needs, as contraction elements 0..3 and 4..7, tokens 16kk + 4h + 0..3 and
   // 16kk + 8 + 4h + 0..3 of dim 32t + lane % 32 (the token order P^T has in its registers): two
@@ -216,6 +228,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     // are masked).
     const int wave_half = wave & 1;
     const char* wave_pool = (const char*)(wave_is_v ? vp : kp);
+    const char* wave_plain = wave_pool - kLoadBias;  // base of plain loads: the per-lane offsets carry the bias
     const uint32_t wave_lds = __builtin_amdgcn_readfirstlane(lds_address(lds)) + (wave_is_v ? Sh::kTileBytes : 0) +
                               wave_half * 16 * kRowBytes;
     // pool row of this wave's half of tile i (uniform pages, tile inside the visible range); read
@@ -231,15 +244,14 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     auto issue = [&](int i, long long row) __attribute__((always_inline)) {
       const uint32_t dst = wave_lds + ring_slot(i) * Sh::kBufferBytes;
       if (tile_is_plain(i)) {
-        const char* base = wave_pool + row * row_bytes;
+        const char* base = wave_plain + row * row_bytes;
         issue_plain(base, dst);
       } else {
         const int t0 = tok_begin + i * kWideTokens + 16 * wave_half;
 #pragma unroll
         for (int u = 0; u < kL; ++u) {
-          const int r = u * Sh::kRowsPerLoad + ld_row0;
-          const int t = min(t0 + r, t_last);
-          const int piece = 16 * (ld_x0 ^ ld_swz(u * Sh::kRowsPerLoad));
+          const int t = min(t0 + ld_row(u), t_last);
+          const int piece = 16 * ld_piece(u);
           load_to_lds(wave_pool + kv_slot(a.kv_indices, kv_begin, t, P, slots) * row_bytes + piece, dst + u * 1024);
         }
       }
@@ -397,7 +409,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       const int page = ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + (t >> p_shift)];
       const int zero = ring_barrier_zero<(kWideAhead - 1) * kL>();
       const uint32_t dst = wave_lds + ring_slot(k + kWideAhead) * Sh::kBufferBytes;
-      const char* base = wave_pool + row * row_bytes;
+      const char* base = wave_plain + row * row_bytes;
       issue_plain(base, dst);
       row_ahead = ((long long)(page + zero) << p_shift) + (t & (P - 1));
     };
@@ -416,7 +428,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     auto read_k = [&](int tile) __attribute__((always_inline)) {
       const char* kt = lds + ring_slot(tile) * Sh::kBufferBytes;
 #pragma unroll
-      for (int s = 0; s < kSteps; ++s) kf[s] = *(const va_u32x4*)(kt + k_row_byte + 16 * ((2 * s + h) ^ swz_j));
+      for (int s = 0; s < kSteps; ++s) kf[s] = *(const va_u32x4*)(kt + k_lane_byte + 256 * s);
     };
     auto score_step = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
