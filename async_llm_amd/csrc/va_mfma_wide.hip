@@ -106,7 +106,17 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   const char* lds = (const char*)smem;
 
   // workgroup -> (slot, kv head); the slot's items are run one after the other
-  const ItemHead where = item_and_head(blockIdx.x, a.num_kv_heads);
+  // The slots of a die run in groups of up to 32 under ONE kv head at a time (a die has 32 compute
+  // units): neighbouring slots hold neighbouring query tiles of one request, which walk the same
+  // K/V rows, so the die's L2 holds one head's stream at a time instead of all of them.
+  ItemHead where;
+  {
+    const unsigned die = blockIdx.x & 7u, turn = blockIdx.x >> 3, per_die = gridDim.x / (8u * a.num_kv_heads);
+    unsigned g = 32;
+    while (per_die % g) g >>= 1;
+    const unsigned block = turn / (g * a.num_kv_heads), within = turn % (g * a.num_kv_heads);
+    where = ItemHead{(int)((block * g + within % g) * 8u + die), (int)(within / g)};
+  }
   const int item_begin = a.wide_slots[where.item], item_end = a.wide_slots[where.item + 1];
   const int hk = where.head;
   const int G = a.num_q_heads / a.num_kv_heads;
