@@ -43,11 +43,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # carried here together with the digest of the kernel sources they were measured on
 # (csrc_digest()), and are reported only while that digest is the one of the sources in the tree.
 MEASURED_TRAFFIC = {
-    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_158_720 + 8_980) + 1024 * (17_894 + 512), "csrc": "857e80c6bc4d551e"},
-    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_630 + 4_712) + 1024 * (9_303 + 64), "csrc": "857e80c6bc4d551e"},
-    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 7_293_081 + 1024 * 131_155, "csrc": "857e80c6bc4d551e"},
-    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (2_526_499 + 1_628_231 + 25_408) + 1024 * (49_781 + 7_078 + 10_368),
-                              "csrc": "857e80c6bc4d551e"},
+    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_159_144 + 8_980) + 1024 * (17_894 + 512), "csrc": "49b4cd49f5849937"},
+    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_644 + 4_712) + 1024 * (9_303 + 64), "csrc": "49b4cd49f5849937"},
+    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_570_221 + 1024 * 131_414, "csrc": "49b4cd49f5849937"},
+    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (2_520_160 + 1_628_332 + 25_407) + 1024 * (49_781 + 7_078 + 10_368),
+                              "csrc": "49b4cd49f5849937"},
 }
 
 
