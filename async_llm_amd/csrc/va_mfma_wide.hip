@@ -21,9 +21,11 @@
 // The loop is a hand-ordered software pipeline: the scores of tile i + 1 run on the matrix pipe
 // under the exponentials of tile i, the products of tile i under the maxima and the score
 // transform of tile i + 1.  Interior tiles of a link take a branch-free ring step.
-// LDS rows are unpadded and swizzled (piece c of tile row r at position c ^ swz(r)), see
-// va_mfma_stream.hip.  The query tile is rotated by all 256 threads, one row block of every wave
-// (128 rows) at a time, into the two ring buffers that are not yet in use.
+// V tiles and the staged query tile keep whole rows in LDS, unpadded and swizzled (piece c of row r
+// at position c ^ swz(r)); K tiles land in fragment order (8-token x 128-byte blocks, see the load
+// pattern in the kernel), so that the K reads of a tile share one address register.  The query tile
+// is rotated by all 256 threads, one row block of every wave (128 rows) at a time, into the two
+// ring buffers that are not yet in use.
 #include <hip/hip_runtime.h>
 
 #include "va_internal.h"

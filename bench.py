@@ -43,11 +43,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # carried here together with the digest of the kernel sources they were measured on
 # (csrc_digest()), and are reported only while that digest is the one of the sources in the tree.
 MEASURED_TRAFFIC = {
-    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_159_144 + 8_980) + 1024 * (17_894 + 512), "csrc": "49b4cd49f5849937"},
-    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_644 + 4_712) + 1024 * (9_303 + 64), "csrc": "49b4cd49f5849937"},
-    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_570_221 + 1024 * 131_414, "csrc": "49b4cd49f5849937"},
-    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (2_520_160 + 1_628_332 + 25_407) + 1024 * (49_781 + 7_078 + 10_368),
-                              "csrc": "49b4cd49f5849937"},
+    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_159_178 + 8_980) + 1024 * (17_893 + 512), "csrc": "dbb28187ddcf157d"},
+    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_633 + 4_712) + 1024 * (9_302 + 64), "csrc": "dbb28187ddcf157d"},
+    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_579_922 + 1024 * 131_424, "csrc": "dbb28187ddcf157d"},
+    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (2_519_998 + 1_628_199 + 25_407) + 1024 * (49_814 + 7_077 + 10_368),
+                              "csrc": "dbb28187ddcf157d"},
 }
 
 
