@@ -8,8 +8,9 @@ batched bf16 decode configuration (64 requests, 16 q / 4 kv heads, head_dim 256,
 page size 16, every view = one shared 8192-token block + 1-3 private blocks of
 256..8192 tokens) and carries, under ``configs``, the same measurements for the
 view-conditioned prefill, the mixed continuous batch, the long-context mRoPE
-decode and the fp32 plumbing case; with ``--workload`` only that workload is
-measured.  Inputs are resident in HBM before the timed region; successive steps
+decode and the fp32 plumbing case, each measured by a child process of its own
+(a fresh allocator and address space, as when the workload is run alone); with
+``--workload`` only that workload is measured, in this process.  Inputs are resident in HBM before the timed region; successive steps
 rotate over several copies of the KV pool so the 256 MB last-level cache cannot
 hold the working set.  Prints ONE JSON line.
 
@@ -26,6 +27,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import subprocess
 import sys
 import time
 
@@ -436,7 +438,7 @@ def measure(wl, steps, warmup, layers, cpu_sample, with_cpu, traffic_ok):
     return line
 
 
-SECONDARY = ("view_prefill", "mixed_batch", "mrope_decode", "plumbing_decode")
+SECONDARY = ("mrope_decode", "mixed_batch", "view_prefill", "plumbing_decode")
 
 
 def main() -> int:
@@ -446,6 +448,53 @@ def main() -> int:
               "no sharding); run with --gpus 1", file=sys.stderr)
         return 2
     import torch
+
+    everything = args.workload is None
+    if everything:
+        # The default run reports every configuration: the batched decode as the line itself, the
+        # others under "configs".  Each is measured by a child process of its own (this one never
+        # touches the GPU): a configuration then sees the allocator and the address space of a fresh
+        # process, as it does when it is run alone or under the profiler, whatever ran before it.
+        if torch.cuda.device_count() < 1:
+            print("bench.py needs a GPU", file=sys.stderr)
+            return 2
+        line = None
+        for name in ("batched_decode",) + SECONDARY:
+            cmd = [sys.executable, os.path.abspath(__file__), "--workload", name,
+                   "--layers", str(1 if name == "plumbing_decode" else args.layers)]
+            if args.kernel:
+                cmd += ["--kernel", args.kernel]
+            if name == "batched_decode":
+                steps, warmup = args.steps, args.warmup
+                cmd += ["--cpu-sample", str(args.cpu_sample)]
+            else:
+                steps, warmup = (None if name == "plumbing_decode" else max(20, args.steps or 20)), None
+            if steps is not None:
+                cmd += ["--steps", str(steps)]
+            if warmup is not None:
+                cmd += ["--warmup", str(warmup)]
+            if args.no_cpu_baseline:
+                cmd += ["--no-cpu-baseline"]
+            child = subprocess.run(cmd, stdout=subprocess.PIPE, text=True)
+            rows = [r for r in child.stdout.splitlines() if r.startswith("{")]
+            if child.returncode != 0 or not rows:
+                print("bench.py: measuring %s failed (exit code %d)" % (name, child.returncode), file=sys.stderr)
+                return child.returncode or 1
+            sub = json.loads(rows[-1])
+            if line is None:
+                line = sub
+                line["configs"] = {}
+                continue
+            line["configs"][name] = {
+                "metric": sub["metric"], "value": sub["value"], "unit": sub["unit"], "dtype": sub["dtype"],
+                "steps": sub["steps"], "warmup": sub["warmup"], "ms_per_step": sub["ms_per_step"],
+                "alg_bytes": sub["config"]["alg_bytes"], "alg_flops": sub["config"]["alg_flops"],
+                "rows": sub["config"]["rows"], "work_items": sub["config"]["work_items"],
+                "wide_items": sub["config"]["wide_items"], "partials": sub["config"]["partials"],
+                "host_prepare_ms": sub["config"]["host_prepare_ms"], "roofline": sub["roofline"],
+                "cpu_baseline": sub.get("cpu_baseline")}
+        print(json.dumps(line), flush=True)
+        return 0
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -459,31 +508,10 @@ def main() -> int:
         return copy_calibration(dev, args.steps)
     if args.workload == "block_merge":
         return block_merge(dev, args.steps, args.warmup, args.layers, not args.no_cpu_baseline)
-    # the default run reports every configuration: the batched decode as the line itself, the others
-    # under "configs"; naming a workload measures that one alone (what the profiler runs do)
-    everything = args.workload is None
-    name = args.workload or "batched_decode"
+    # naming a workload measures that one alone, in this process (what the profiler runs do)
     traffic_ok = args.layers == 4 and not os.environ.get("VIEWATTN_PLAN")
-    wl = build_workload(name, dev, args.layers, args.kernel)
+    wl = build_workload(args.workload, dev, args.layers, args.kernel)
     line = measure(wl, args.steps, args.warmup, args.layers, args.cpu_sample, not args.no_cpu_baseline, traffic_ok)
-    del wl
-    if everything:
-        line["configs"] = {}
-        for other in SECONDARY:
-            torch.cuda.empty_cache()
-            layers = 1 if other == "plumbing_decode" else args.layers
-            wl = build_workload(other, dev, layers, args.kernel)
-            sub = measure(wl, None if other == "plumbing_decode" else max(20, args.steps or 20), None, layers, 0,
-                          not args.no_cpu_baseline, traffic_ok)
-            del wl
-            line["configs"][other] = {
-                "metric": sub["metric"], "value": sub["value"], "unit": sub["unit"], "dtype": sub["dtype"],
-                "steps": sub["steps"], "warmup": sub["warmup"], "ms_per_step": sub["ms_per_step"],
-                "alg_bytes": sub["config"]["alg_bytes"], "alg_flops": sub["config"]["alg_flops"],
-                "rows": sub["config"]["rows"], "work_items": sub["config"]["work_items"],
-                "wide_items": sub["config"]["wide_items"], "partials": sub["config"]["partials"],
-                "host_prepare_ms": sub["config"]["host_prepare_ms"], "roofline": sub["roofline"],
-                "cpu_baseline": sub.get("cpu_baseline")}
     print(json.dumps(line), flush=True)
     return 0
 
