@@ -206,7 +206,16 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
         const long long src_row = indirect ? (long long)a.qref_rows[qref + iq] : a.sub_worker[subrow];
         const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
         const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
-        rotated_query_unit<E>(a.rope, qh, x, p, c0, c1, p0, p1);
+        if (a.rope.mode == VA_ROPE_TABLE && x < a.rope.rotary_dim / 16) {
+          // the table entries of the unit in four 16-byte loads
+          TableQueryUnit<E> unit;
+          unit.load(a.rope, qh, x, p);
+          unit.finish(a.rope, p, p0, p1);
+          c0 = x;
+          c1 = x + a.rope.rotary_dim / 16;
+        } else {
+          rotated_query_unit<E>(a.rope, qh, x, p, c0, c1, p0, p1);
+        }
       }
       q_stage[jr * kChunks + (c0 ^ swz<kD>(jr))] = va_u32x4{p0.x, p0.y, p0.z, p0.w};
       q_stage[jr * kChunks + (c1 ^ swz<kD>(jr))] = va_u32x4{p1.x, p1.y, p1.z, p1.w};

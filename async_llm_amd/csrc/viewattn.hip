@@ -158,10 +158,30 @@ __global__ __launch_bounds__(256) void rope_store_vec_kernel(
     xa.raw = *(const uint4*)(xr + ea);
     xb.raw = *(const uint4*)(xr + eb);
     const Pos3 p = load_pos(pos, pos_axis_stride, row);
+    float cs[kVec], sns[kVec];
+    if (rope.mode == VA_ROPE_TABLE) {
+      // the kVec cosines and sines of this piece in 16-byte loads (the launcher has checked the table's alignment)
+      long long a = p.t < 0 ? -p.t : p.t;
+      if (a > rope.max_pos - 1) a = rope.max_pos - 1;
+      const float* trow = rope.cos_sin + a * (long long)rope.rotary_dim + i0;
+#pragma unroll
+      for (int k = 0; k < kVec; k += 4) {
+        const float4 c4 = *(const float4*)(trow + k), s4 = *(const float4*)(trow + rope.half + k);
+        cs[k] = c4.x, cs[k + 1] = c4.y, cs[k + 2] = c4.z, cs[k + 3] = c4.w;
+        sns[k] = s4.x, sns[k + 1] = s4.y, sns[k + 2] = s4.z, sns[k + 3] = s4.w;
+      }
+      if (p.t < 0) {
+#pragma unroll
+        for (int k = 0; k < kVec; ++k) sns[k] = -sns[k];
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < kVec; ++k) rope_cos_sin(rope, p, i0 + k, cs[k], sns[k]);
+    }
 #pragma unroll
     for (int k = 0; k < kVec; ++k) {
-      float c, sn, y1, y2;
-      rope_cos_sin(rope, p, i0 + k, c, sn);
+      float y1, y2;
+      const float c = cs[k], sn = sns[k];
       rope_pair<E>(rope, c, sn, E::load(xa.e[k]), E::load(xb.e[k]), y1, y2);
       ya.e[k] = E::store(y1);
       yb.e[k] = E::store(y2);
@@ -188,8 +208,10 @@ int launch_rope_store(const void* x, const void* v, void* y, void* v_out, long l
   auto piecewise = [&](const void* ptr, long long stride) {
     return ptr == nullptr || ((uintptr_t)ptr % 16 == 0 && stride % kVec == 0);
   };
+  const bool table_ok = rope.mode != VA_ROPE_TABLE || (kVec % 4 == 0 && (uintptr_t)rope.cos_sin % 16 == 0 &&
+                                                      rope.rotary_dim % 4 == 0 && rope.half % 4 == 0);
   const bool vec = head_dim % kVec == 0 && rope.half % kVec == 0 && piecewise(x, x_stride) && piecewise(y, y_stride) &&
-                   piecewise(v, v_stride) && piecewise(v_out, y_stride);
+                   piecewise(v, v_stride) && piecewise(v_out, y_stride) && table_ok;
   if (vec) {
     const bool copy_tail = x != y || dst != nullptr;
     const int pair_units = n_heads * (rope.half / kVec);

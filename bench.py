@@ -45,11 +45,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # carried here together with the digest of the kernel sources they were measured on
 # (csrc_digest()), and are reported only while that digest is the one of the sources in the tree.
 MEASURED_TRAFFIC = {
-    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_159_178 + 8_980) + 1024 * (17_893 + 512), "csrc": "dbb28187ddcf157d"},
-    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_633 + 4_712) + 1024 * (9_302 + 64), "csrc": "dbb28187ddcf157d"},
-    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_579_922 + 1024 * 131_424, "csrc": "dbb28187ddcf157d"},
-    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (2_519_998 + 1_628_199 + 25_407) + 1024 * (49_814 + 7_077 + 10_368),
-                              "csrc": "dbb28187ddcf157d"},
+    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_162_281 + 8_981) + 1024 * (17_894 + 512), "csrc": "87cf5f3ac8ad1a0f"},
+    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_647 + 4_712) + 1024 * (9_303 + 64), "csrc": "87cf5f3ac8ad1a0f"},
+    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_587_516 + 1024 * 131_434, "csrc": "87cf5f3ac8ad1a0f"},
+    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (2_522_692 + 1_628_647 + 25_407) + 1024 * (49_816 + 7_078 + 10_368),
+                              "csrc": "87cf5f3ac8ad1a0f"},
 }
 
 
