@@ -327,11 +327,12 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   // Narrow tiles of chains (the last rows of a request) are cut by the same budget, one item a piece.
   const int64_t slots_wanted = std::max(1, 256 / shape->num_kv_heads);
   int64_t chain_budget = INT64_MAX;
-  // A piece stages its query tile again, which costs a wide tile about as much as walking this many
-  // tokens: the packing charges it to the slot's room, makes no piece shorter than it, and keeps a
-  // tile's remainder under it with the piece before.
-  const int32_t piece_cost = 6 * gran;
-  const int32_t min_piece = piece_cost;
+  // A piece of a wide tile stages its query tile once per segment of the view it walks (the query is
+  // rotated for every block anew), which costs about as much as walking `seg_cost` tokens: the packing
+  // charges every (piece, segment) to the slot's room.  A tile's remainder that would cost less than
+  // `min_piece` stays with the piece before it.
+  const int32_t seg_cost = 10 * gran;
+  const int32_t min_piece = 6 * gran;
   if (chain_tiles > 0 && chain_tiles < 4 * slots_wanted) {
     // (at most `want` <= target cuts are made, which is what bounds a fixed-capacity plan)
     const int64_t want = std::max<int64_t>(1, std::min<int64_t>(target, slots_wanted));
@@ -347,19 +348,26 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   // over (a tile's short remainder kept with the piece before it) is made up for by the slots after
   // it, and their number never exceeds the number wanted.
   const int32_t slot_room = pack ? round_up(chain_budget + (align_cuts ? 15 : 0), gran) : 0;  // narrow tiles of chains
-  int64_t wide_tiles = 0;
-  for (auto& ch : chains) {
-    cut_tiles(s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]], tiles);
-    for (auto& tl : tiles) wide_tiles += tl.second - tl.first > q_tile;
+  int64_t wide_segments = 0;  // (wide tile, visible segment) pairs
+  if (pack) {
+    for (auto& ch : chains) {
+      const int32_t nq = s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]];
+      cut_tiles(nq, tiles);
+      for (auto& tl : tiles) {
+        if (tl.second - tl.first <= q_tile) continue;
+        for (int32_t m : ch) wide_segments += visible_end(s->seq_lens[m], nq, s->flags[m] & VA_SUB_CAUSAL, tl.second) > 0;
+      }
+    }
   }
   int64_t slots_left = pack ? std::max<int64_t>(1, (wide_chain_tokens + chain_budget - 1) / chain_budget) : 0;
-  // what is still to be placed, set-ups included: a piece per slot or per tile, whichever are more,
-  // and another for about every other of those that are fewer (where a slot boundary falls inside a tile)
-  int64_t wide_left = wide_chain_tokens +
-                      piece_cost * (std::max(wide_tiles, slots_left) + std::min(wide_tiles, slots_left) / 2);
+  // What is still to be placed, set-ups included: every segment of every tile, and one more for every
+  // slot boundary (it falls inside some segment, which is then staged on both sides).  An estimate
+  // on the high side leaves the LAST slot short, one on the low side would leave it long -- and the
+  // longest slot is the time of the launch.
+  int64_t wide_left = wide_chain_tokens + seg_cost * (wide_segments + slots_left - 1);
   auto next_wide_room = [&]() -> int32_t {
     if (slots_left <= 1) return INT32_MAX;  // the last slot takes whatever is left
-    const int64_t share = (wide_left + slots_left - 1) / slots_left;
+    const int64_t share = std::max<int64_t>((wide_left + slots_left - 1) / slots_left, seg_cost + min_piece);
     --slots_left;
     return round_up(share + (align_cuts ? 15 : 0), 16);
   };
@@ -392,26 +400,20 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
       // Cut the tile's walk where the room of the current budget ends.  Wide tiles fill the shared
       // slots (the room carries over from tile to tile); a narrow tile starts a budget of its own.
       int32_t room = wide ? wide_room : slot_room;
+      const int32_t seg = wide ? seg_cost : 0;  // what starting a segment in a piece costs
       auto next_room = [&]() {
         if (wide) ++wide_slot;
         room = wide ? next_wide_room() : slot_room;
       };
-      auto next_piece_room = [&]() {  // a further piece of this tile, in the next slot
-        next_room();
-        if (wide) {
-          room -= std::min(room, piece_cost);
-          wide_left -= piece_cost;
-        }
-      };
-      if (wide && room < piece_cost + min_piece) next_room();  // too little left for a piece worth its set-up
-      if (wide) {  // the set-up of the tile's first piece
-        room -= piece_cost;
-        wide_left -= piece_cost;
-      }
-      int64_t left = tile_tokens;  // tokens of the tile not yet in a piece
-      // no tiny last piece: a remainder under min_piece stays with the piece before it
+      if (wide && room < seg + min_piece) next_room();  // too little left for a piece worth its set-up
+      int64_t left = tile_tokens;            // tokens of the tile not yet in a piece
+      int64_t segs_left = (int64_t)all.size();  // segments of the tile not yet finished
+      // no tiny last piece: a remainder that would cost less than `small` stays with the piece before it
+      // (small next to a slot's share: the slot that keeps it runs that much longer than the others)
+      const int64_t small = wide ? std::min<int64_t>(min_piece + seg, chain_budget / 8) : min_piece;
       auto fit_room = [&]() {
-        if (left > room && left - room < min_piece) room = (int32_t)left;
+        const int64_t need = left + seg * segs_left;  // room that takes all that is left
+        if (need > room && need - room < small - seg) room = (int32_t)need;
       };
       fit_room();
       std::vector<Link> cur;
@@ -422,29 +424,36 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
       for (auto l : all) {
         const bool aligned = align_cuts && !(l.flags & VA_LINK_SLOTS);
         while (l.tok_begin < l.tok_end) {
-          int32_t take = std::min(room, l.tok_end - l.tok_begin);
-          if (aligned && take < l.tok_end - l.tok_begin) {
-            take = take / 16 * 16;  // l.tok_begin is a multiple of 16: segments start at 0, cuts keep it so
-            if (take == 0) {        // under 16 tokens of room left: the piece ends here
-              close_piece();
-              next_piece_room();
-              fit_room();
+          int32_t take = room > seg ? std::min(room - seg, l.tok_end - l.tok_begin) : 0;
+          if (aligned && take < l.tok_end - l.tok_begin) take = take / 16 * 16;  // l.tok_begin is a multiple of 16: segments start at 0, cuts keep it so
+          if (take <= 0) {  // no room left to start (or go on with) the segment here: the piece ends
+            if (!cur.empty() && left + seg * segs_left < small) {  // ... unless what is left is too little for a piece of its own
+              room = (int32_t)(left + seg * segs_left);
               continue;
             }
+            close_piece();
+            next_room();
+            fit_room();
+            continue;
           }
           Link piece = l;
           piece.tok_end = l.tok_begin + take;
           cur.push_back(piece);
           l.tok_begin += take;
           left -= take;
-          room -= take;
-          if (wide) wide_left -= take;
+          room -= take + seg;
+          if (wide) wide_left -= take + seg;
           if (room <= 0 && left > 0) {
+            if (left + seg * segs_left < small) {  // too little for a piece of its own: it stays with this one
+              room = (int32_t)(left + seg * segs_left);
+              continue;
+            }
             close_piece();
-            next_piece_room();
+            next_room();
             fit_room();
           }
         }
+        --segs_left;
       }
       close_piece();
       if (wide) {

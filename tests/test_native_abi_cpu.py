@@ -315,47 +315,64 @@ def test_compute_entry_points_refuse_cpu_tensors():
         apply_rope_correction(torch.zeros(2, 1, 8), torch.zeros(2, dtype=torch.int64), torch.zeros(4, 8))
 
 
-def test_few_wide_tiles_are_packed_into_slots_of_equal_length():
-    """Four prefill chunks of 64 tokens (two wide tiles each at 16 q / 4 kv heads of 256 dims) over
-    views of 1.5k to 30k tokens: 8 tiles cannot fill 64 workgroup slots per kv head, and cut one
-    by one into similar pieces they would still fill them unevenly.  The planner lays all walks
-    end to end and gives every slot the same share; a slot holds the end of one tile and the start
-    of the next."""
+def _packed_slot_loads(chunk_tokens, views, coverage=True):
+    """Plan prefill chunks of `chunk_tokens` new tokens, one per entry of `views` (the lengths of the
+    context segments of the chunk's view; its own block holds 100 tokens before the chunk), at
+    16 q / 4 kv heads of 256 dims.  Returns (counts, total tokens walked, per-slot loads): a slot's
+    load is the tokens it walks plus the set-up of every (piece, segment) it holds, worth ~640 tokens."""
     page = 16
     qo, kvp, kvi, lens, flags, chain, sw = [0], [0], [], [], [], [], []
     n_rows = 0
-    for r, context in enumerate((30000, 1500, 12345, 22222)):
-        rows = list(range(n_rows, n_rows + 64))
-        n_rows += 64
-        for L in (512, context):
+    for r, segments in enumerate(views):
+        rows = list(range(n_rows, n_rows + chunk_tokens))
+        n_rows += chunk_tokens
+        for L in segments:
             kvi += list(range(len(kvi), len(kvi) + -(-L // page)))
             kvp.append(len(kvi)); lens.append(L); flags.append(0); chain.append(r)
             sw += rows; qo.append(len(sw))
-        kvi += list(range(len(kvi), len(kvi) + -(-(100 + 64) // page)))
-        kvp.append(len(kvi)); lens.append(164); flags.append(1); chain.append(r)
+        kvi += list(range(len(kvi), len(kvi) + -(-(100 + chunk_tokens) // page)))
+        kvp.append(len(kvi)); lens.append(100 + chunk_tokens); flags.append(1); chain.append(r)
         sw += rows; qo.append(len(sw))
     rc, blob, counts = build_plan(qo, kvp, kvi, lens, flags, chain, sw, n_rows, heads=(16, 4, 256), page=page,
                                   dtype=native.VA_BF16, kernel=native.VA_KERNEL_MFMA)
     assert rc == 0
-    check_coverage(blob, qo, kvp, lens, flags, sw, n_rows)
+    if coverage:  # (every visible pair once: a check of rows x tokens steps in Python)
+        check_coverage(blob, qo, kvp, lens, flags, sw, n_rows)
     h, items, links, *_ = decode_plan(blob)
     slots = blob[h[H["OFF_WIDE_SLOTS"]]: h[H["OFF_WIDE_SLOTS"]] + h[H["N_WIDE_SLOTS"]] + 1]
     assert counts.n_wide_slots == h[H["N_WIDE_SLOTS"]] == 64 and counts.n_wide_items >= 64
-    total = 2 * (4 * 512 + 30000 + 1500 + 12345 + 22222) + sum(2 * 100 + 32 + 64 for _ in range(4))
-    assert int(items[: slots[-1], 4].sum()) == total
-    # a slot's load: the tokens it walks plus the set-up of each of its pieces (worth ~384 tokens)
-    load = [int(items[a:b, 4].sum()) + 384 * int(b - a) for a, b in zip(slots, slots[1:])]
-    mean = sum(load) / 64
-    # the longest slot sets the time of the launch (the last slot takes what is left and may be short)
-    assert max(load) <= 1.06 * mean and min(load) > 0 and sorted(load)[1] >= 0.9 * mean, (min(load), max(load), mean)
-    assert min(int(it[4]) for it in items[: slots[-1]]) >= 384 - 16  # no piece too short to be worth its set-up
+    loads = [int(items[a:b, 4].sum()) + 640 * int(items[a:b, 1].sum()) for a, b in zip(slots, slots[1:])]
+    # no piece too small to be worth a set-up of its own: at least ~384 tokens + a segment's 640, unless
+    # the slots themselves are so small that a remainder of that size would unbalance them (an eighth of a slot)
+    assert min(int(it[4]) + 640 * int(it[1]) for it in items[: slots[-1]]) >= min(384 + 640, sum(loads) // 64 // 8) - 16
+    return counts, int(items[: slots[-1], 4].sum()), loads
+
+
+def test_few_wide_tiles_are_packed_into_slots_of_equal_length():
+    """Prefill chunks whose wide tiles (32 tokens x 4 heads each) cannot fill 64 workgroup slots per
+    kv head evenly: views of 1.5k to 30k tokens, and cut one by one into similar pieces the tiles
+    would still fill the slots unevenly.  The planner lays all walks end to end and gives every
+    slot the same share, set-ups included; a slot holds the end of one tile and the start of the
+    next.  The longest slot is the time of the launch (one workgroup per CU, one round): it must
+    stay close to the mean, and no slot may be left to take a long remainder."""
+    # 8 tiles for 64 slots: every tile is cut in about eight
+    counts, total, loads = _packed_slot_loads(64, [(512, 30000), (512, 1500), (512, 12345), (512, 22222)])
+    assert total == 2 * (4 * 512 + 30000 + 1500 + 12345 + 22222) + sum(2 * 100 + 32 + 64 for _ in range(4))
+    # the longest slot is the time of the launch; slots at the end may be short or empty
+    assert sum(loads) >= 0.92 * 64 * max(loads), (min(loads), max(loads), sum(loads) / 64)
+    # 64 tiles for 64 slots (four chunks of 512 tokens over views of two to five blocks): most slots hold the
+    # end of one tile and the start of the next
+    views = [(512, 9000, 14000), (512, 2500), (512, 7000, 8000, 9000, 6000), (512, 900, 11000, 3000)]
+    counts, total, loads = _packed_slot_loads(512, views, coverage=False)
+    assert total == sum(16 * (sum(v) + 100) + sum(range(32, 513, 32)) for v in views)
+    assert sum(loads) >= 0.96 * 64 * max(loads) and min(loads) > 0, (min(loads), max(loads), sum(loads) / 64)
 
 
 def test_prefill_tiles_are_cut_by_tokens_on_page_group_boundaries():
     """Two prefill requests of one 32-row tile each, one over 30000 context tokens
     in three segments of odd lengths, one over 700: too few tiles to fill the
     machine, so the planner splits them by tokens.  The long tile must come out
-    in many pieces of similar weight, the short one whole; with pages of 16
+    in many pieces of similar weight, the short one in at most three; with pages of 16
     tokens every cut inside a segment lies on a 16-token boundary, with pages of
     4 it need not; every visible pair is covered once either way."""
     for page in (16, 4):
@@ -380,10 +397,13 @@ def test_prefill_tiles_are_cut_by_tokens_on_page_group_boundaries():
         weight = {}
         for it in real:
             ls = links[it[0]: it[0] + it[1]]
-            tokens = sum(int(l[2] - l[1]) for l in ls)
+            # what a piece costs its workgroup: the tokens it walks and ~640 more for every segment it stages
+            tokens = sum(int(l[2] - l[1]) for l in ls) + 640 * len(ls)
             long_one = any(int(l[0]) < kvp[3] for l in ls)  # kv_begin inside the first request's tables
             weight.setdefault(long_one, []).append(tokens)
-        assert len(weight[False]) == 1, "the short tile was cut"
+        # (the short tile, 748 tokens in two segments, is worth about two slots' shares with its set-ups:
+        # it may be cut once or twice, not shredded)
+        assert len(weight[False]) <= 3, "the short tile was cut in many pieces"
         assert len(weight[True]) >= 20, "the long tile was not cut by its tokens"
         assert max(weight[True]) <= 1.3 * sorted(weight[True])[1], weight[True]  # (one piece takes what is left)
         inner = [int(l[1]) for it in real for l in links[it[0]: it[0] + it[1]] if l[1] > 0]
