@@ -343,123 +343,247 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   // tokens or more: a piece that starts on such a boundary is fetched with uniform loads)
   const bool align_cuts = shape->page_size >= 16 && (shape->page_size & (shape->page_size - 1)) == 0;
   const bool pack = chain_budget != INT64_MAX;
-  // The room of a new wide slot is the even share of what is still to be placed over the slots
-  // still to be opened, so that a slot closed early (less than min_piece of its room left) or run
-  // over (a tile's short remainder kept with the piece before it) is made up for by the slots after
-  // it, and their number never exceeds the number wanted.
   const int32_t slot_room = pack ? round_up(chain_budget + (align_cuts ? 15 : 0), gran) : 0;  // narrow tiles of chains
-  int64_t wide_segments = 0;  // (wide tile, visible segment) pairs
+
+  // Wide tiles are packed in LOCKSTEP BUNDLES.  The query tiles of one chunk all stream the chunk's
+  // view; packed one after the other into slots they would walk it at different places at any one
+  // time, and each would fetch it from HBM for itself.  So the workgroup slots are taken in groups of
+  // `lanes` (the slots that run side by side on one die), up to `lanes` neighbouring tiles of a chain
+  // form a bundle, and a bundle's walk is cut ONCE, for all its tiles alike: the lanes of a group walk
+  // the same tokens at the same time, one of them fetches a K/V tile from HBM and the others find
+  // it in the die's L2.  A bundle of m <= lanes / 2 tiles has its walk cut into f = lanes / m parts
+  // that run side by side (lane = part * m + tile), so a short chain still fills the group.
+  const int64_t want_slots = pack ? std::max<int64_t>(1, std::min<int64_t>(target, slots_wanted)) : 1;
+  const int32_t lanes = (int32_t)std::max<int64_t>(1, want_slots / kXcds);
+  const int32_t groups_wanted = (int32_t)std::min<int64_t>(want_slots, kXcds);
+  struct Bundle {
+    int32_t first = 0, m = 0, f = 1;  // tiles [first, first + m) of the chain; f parts side by side
+    int32_t part = 0;                 // walk positions per part
+    std::vector<int32_t> subs;        // the chain members any tile of the bundle sees
+    std::vector<int32_t> off;         // walk position of each member's first token
+    std::vector<int32_t> starts;      // positions within a part where some lane starts a member (sorted)
+    // What positions [x0, x1) cost the slowest lane of the bundle: its tokens, and a set-up (worth
+    // `seg` tokens) for the segment it is in at x0 and for every member that starts inside its range.
+    int64_t cost(int64_t x0, int64_t x1, int32_t seg) const {
+      int64_t most = 0;
+      for (int32_t g = 0; g < f; ++g) {
+        int64_t n = 1;
+        for (int32_t o : off) {
+          const int64_t x = (int64_t)o - (int64_t)g * part;
+          n += x > x0 && x < x1;
+        }
+        most = std::max(most, n);
+      }
+      return (x1 - x0) + seg * most;
+    }
+  };
+  auto make_bundle = [&](const std::vector<int32_t>& ch, int32_t nq, int32_t first, int32_t m) {
+    Bundle bd;
+    bd.first = first;
+    bd.m = m;
+    const int32_t b_last = tiles[first + m - 1].second;  // the last tile sees most
+    int64_t pos = 0;
+    for (int32_t sub : ch) {
+      const int32_t vis = visible_end(s->seq_lens[sub], nq, s->flags[sub] & VA_SUB_CAUSAL, b_last);
+      if (vis <= 0) continue;
+      bd.subs.push_back(sub);
+      bd.off.push_back((int32_t)pos);
+      pos += align_cuts ? round_up(vis, 16) : vis;  // every member starts at a multiple of 16: so do all cuts within it
+    }
+    if (pos == 0) return bd;
+    bd.f = (int32_t)std::max<int64_t>(1, std::min<int64_t>(lanes / m, pos / (8 * gran)));
+    bd.part = bd.f == 1 ? (int32_t)pos : round_up((pos + bd.f - 1) / bd.f, 16);
+    for (int32_t g = 0; g < bd.f; ++g)
+      for (int32_t o : bd.off) {
+        const int64_t x = (int64_t)o - (int64_t)g * bd.part;
+        if (x > 0 && x < bd.part) bd.starts.push_back((int32_t)x);
+      }
+    std::sort(bd.starts.begin(), bd.starts.end());
+    bd.starts.erase(std::unique(bd.starts.begin(), bd.starts.end()), bd.starts.end());
+    return bd;
+  };
+  // bundles of a chain's tile list (as cut_tiles left it in `tiles`)
+  auto bundles_of = [&](const std::vector<int32_t>& ch, int32_t nq, std::vector<Bundle>& out_bundles) {
+    out_bundles.clear();
+    int32_t n_wide_tiles = 0;
+    while (n_wide_tiles < (int32_t)tiles.size() && tiles[n_wide_tiles].second - tiles[n_wide_tiles].first > q_tile) ++n_wide_tiles;
+    for (int32_t first = 0; first < n_wide_tiles; first += lanes) {
+      Bundle bd = make_bundle(ch, nq, first, std::min(lanes, n_wide_tiles - first));
+      if (bd.part > 0) out_bundles.push_back(std::move(bd));
+    }
+  };
+  std::vector<Bundle> bundles;
+  int64_t wide_walk = 0, wide_cost = 0;  // positions of all bundles; with their set-ups
   if (pack) {
     for (auto& ch : chains) {
       const int32_t nq = s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]];
       cut_tiles(nq, tiles);
-      for (auto& tl : tiles) {
-        if (tl.second - tl.first <= q_tile) continue;
-        for (int32_t m : ch) wide_segments += visible_end(s->seq_lens[m], nq, s->flags[m] & VA_SUB_CAUSAL, tl.second) > 0;
+      bundles_of(ch, nq, bundles);
+      for (auto& bd : bundles) {
+        wide_walk += bd.part;
+        wide_cost += bd.cost(0, bd.part, seg_cost);
       }
     }
   }
-  int64_t slots_left = pack ? std::max<int64_t>(1, (wide_chain_tokens + chain_budget - 1) / chain_budget) : 0;
-  // What is still to be placed, set-ups included: every segment of every tile, and one more for every
-  // slot boundary (it falls inside some segment, which is then staged on both sides).  An estimate
-  // on the high side leaves the LAST slot short, one on the low side would leave it long -- and the
-  // longest slot is the time of the launch.
-  int64_t wide_left = wide_chain_tokens + seg_cost * (wide_segments + slots_left - 1);
-  auto next_wide_room = [&]() -> int32_t {
-    if (slots_left <= 1) return INT32_MAX;  // the last slot takes whatever is left
-    const int64_t share = std::max<int64_t>((wide_left + slots_left - 1) / slots_left, seg_cost + min_piece);
-    --slots_left;
+  // The room of a new group is the even share of what is still to be placed over the groups still
+  // to be opened, so that a group closed early (less than min_piece of its room left) or run over (a
+  // bundle's short remainder kept with the piece before it) is made up for by the groups after it,
+  // and their number never exceeds the number wanted.
+  const int64_t group_budget = pack ? std::max<int64_t>((wide_walk + groups_wanted - 1) / groups_wanted, 16 * gran) : 0;
+  int64_t groups_left = pack ? std::max<int64_t>(1, (wide_walk + group_budget - 1) / group_budget) : 0;
+  // What is still to be placed, set-ups included: every segment of every bundle, and one more for
+  // every group boundary (it falls inside some segment, which is then staged on both sides).  An
+  // estimate on the high side leaves the LAST group short, one on the low side would leave it long --
+  // and the longest group is the time of the launch.
+  int64_t wide_left = wide_cost + seg_cost * (groups_left - 1);
+  auto next_wide_room = [&]() -> int64_t {
+    if (groups_left <= 1) return INT32_MAX;  // the last group takes whatever is left
+    const int64_t share = std::max<int64_t>((wide_left + groups_left - 1) / groups_left, seg_cost + min_piece);
+    --groups_left;
     return round_up(share + (align_cuts ? 15 : 0), 16);
   };
-  int32_t wide_slot = 0, wide_room = pack ? next_wide_room() : 0;  // the slot being filled with wide pieces
+  int32_t wide_group = 0;                              // the group being filled
+  int64_t wide_room = pack ? next_wide_room() : 0;  // the room left in it: it carries over from bundle to bundle
+  // Cut a bundle's walk where the room of the current group ends; close(x0, x1, group) takes every piece.
+  auto cut_bundle = [&](const Bundle& bd, auto&& close) {
+    // no tiny last piece: a remainder that would cost less than `small` stays with the piece before it
+    // (small next to a group's share: the group that keeps it runs that much longer than the others)
+    const int64_t small = std::min<int64_t>(min_piece + seg_cost, group_budget / 8);
+    int64_t x = 0;
+    while (x < bd.part) {
+      if (wide_room < seg_cost + min_piece) {  // too little left for a piece worth its set-up
+        ++wide_group;
+        wide_room = next_wide_room();
+      }
+      // the furthest end the room pays for: between two starts the cost grows by one per position
+      int64_t x1 = bd.part;
+      if (bd.cost(x, bd.part, seg_cost) > wide_room) {
+        int64_t from = x;  // cost(x, from) fits
+        for (size_t i = 0; i <= bd.starts.size(); ++i) {
+          const int64_t to = i < bd.starts.size() ? bd.starts[i] : bd.part;
+          if (to <= x) continue;
+          const int64_t c = bd.cost(x, to, seg_cost);
+          if (c <= wide_room) {
+            from = to;
+            continue;
+          }
+          x1 = std::max(from, to - (c - wide_room));
+          break;
+        }
+        if (align_cuts) x1 = x1 / 16 * 16;  // x and every start are multiples of 16
+        if (x1 <= x) x1 = std::min<int64_t>(bd.part, x + 16);
+        if (x1 < bd.part && bd.cost(x1, bd.part, seg_cost) < small) x1 = bd.part;
+      }
+      close(x, x1, wide_group);
+      const int64_t c = bd.cost(x, x1, seg_cost);
+      wide_room -= c;
+      wide_left -= c;
+      x = x1;
+    }
+  };
+
+  // Cut a narrow tile's walk (links in walking order) into budgets of `slot_room` tokens, one item a
+  // piece; a remainder of less than min_piece stays with the piece before it.
+  auto cut_walk = [&](const std::vector<Link>& walk, auto&& close) {
+    int32_t room = slot_room;
+    int64_t left = 0;  // tokens of the walk not yet in a piece
+    for (auto& l : walk) left += l.tok_end - l.tok_begin;
+    auto fit_room = [&]() {
+      if (left > room && left - room < min_piece) room = (int32_t)left;
+    };
+    fit_room();
+    std::vector<Link> cur;
+    auto close_piece = [&]() {
+      if (!cur.empty()) close(cur);
+      cur.clear();
+    };
+    for (auto l : walk) {
+      const bool aligned = align_cuts && !(l.flags & VA_LINK_SLOTS);
+      while (l.tok_begin < l.tok_end) {
+        int32_t take = std::min(room, l.tok_end - l.tok_begin);
+        if (aligned && take < l.tok_end - l.tok_begin) take = take / 16 * 16;  // l.tok_begin is a multiple of 16: segments start at 0, cuts keep it so
+        if (take <= 0) {  // no room left to go on here: the piece ends
+          if (!cur.empty() && left < min_piece) {  // ... unless what is left is too little for a piece of its own
+            room = (int32_t)left;
+            continue;
+          }
+          close_piece();
+          room = slot_room;
+          fit_room();
+          continue;
+        }
+        Link piece = l;
+        piece.tok_end = l.tok_begin + take;
+        cur.push_back(piece);
+        l.tok_begin += take;
+        left -= take;
+        room -= take;
+        if (room <= 0 && left > 0) {
+          if (left < min_piece) {  // too little for a piece of its own: it stays with this one
+            room = (int32_t)left;
+            continue;
+          }
+          close_piece();
+          room = slot_room;
+          fit_room();
+        }
+      }
+    }
+    close_piece();
+  };
+
   for (auto& ch : chains) {
     const int32_t nq = s->qo_indptr[ch[0] + 1] - s->qo_indptr[ch[0]];
     cut_tiles(nq, tiles);
-    for (auto& tl : tiles) {
-      const int32_t a = tl.first, b = tl.second;
-      const bool wide = b - a > q_tile;
-      std::vector<Link> all;
-      int64_t tile_tokens = 0;
+    // the links of tile rows [a, b), clipped to walk positions [lo, hi) of a bundle (all of them without one)
+    auto tile_links = [&](int32_t a, int32_t b, const Bundle* bd, int64_t lo, int64_t hi) {
+      std::vector<Link> links;
+      size_t k = 0;
       for (int32_t m : ch) {
         const bool causal = s->flags[m] & VA_SUB_CAUSAL;
         const int32_t len = s->seq_lens[m];
-        const int32_t vis = visible_end(len, nq, causal, b);
-        if (vis <= 0) continue;
+        int32_t t0 = 0, t1 = visible_end(len, nq, causal, b);
+        if (bd) {
+          if (k >= bd->subs.size() || bd->subs[k] != m) continue;  // no tile of the bundle sees this member
+          const int64_t off = bd->off[k++];
+          t0 = (int32_t)(std::max<int64_t>(lo, off) - off);
+          t1 = (int32_t)(std::min<int64_t>(hi, off + t1) - off);
+        }
+        if (t1 <= t0) continue;
         const int32_t cbase = causal ? len - nq + a : VA_NO_CAUSAL;
-        all.push_back(Link{s->kv_indptr[m], 0, vis, s->qo_indptr[m] + a, cbase,
-                           (s->flags[m] & VA_SUB_SLOTS) ? VA_LINK_SLOTS : 0});
-        tile_tokens += vis;
+        links.push_back(Link{s->kv_indptr[m], t0, t1, s->qo_indptr[m] + a, cbase,
+                             (s->flags[m] & VA_SUB_SLOTS) ? VA_LINK_SLOTS : 0});
       }
+      return links;
+    };
+    auto tile_rows = [&](int32_t a, int32_t b) {
       std::vector<int32_t> rows;
       for (int32_t r = a; r < b; ++r) rows.push_back((int32_t)s->sub_worker[s->qo_indptr[ch[0]] + r]);
+      return rows;
+    };
+    if (pack) {
+      bundles_of(ch, nq, bundles);
+      for (auto& bd : bundles) {
+        cut_bundle(bd, [&](int64_t x0, int64_t x1, int32_t group) {
+          for (int32_t g = 0; g < bd.f; ++g)
+            for (int32_t j = 0; j < bd.m; ++j) {
+              const int32_t a = tiles[bd.first + j].first, b = tiles[bd.first + j].second;
+              const std::vector<Link> links = tile_links(a, b, &bd, (int64_t)g * bd.part + x0, (int64_t)g * bd.part + x1);
+              if (!links.empty()) emit(b - a, links, tile_rows(a, b), -1, group * lanes + g * bd.m + j);
+            }
+        });
+      }
+    }
+    for (auto& tl : tiles) {
+      const int32_t a = tl.first, b = tl.second;
+      if (pack && b - a > q_tile) continue;  // packed above
+      const std::vector<Link> all = tile_links(a, b, nullptr, 0, 0);
       if (all.empty()) continue;
       if (!pack) {
-        emit(b - a, all, std::move(rows));
+        emit(b - a, all, tile_rows(a, b));
         continue;
       }
-      // Cut the tile's walk where the room of the current budget ends.  Wide tiles fill the shared
-      // slots (the room carries over from tile to tile); a narrow tile starts a budget of its own.
-      int32_t room = wide ? wide_room : slot_room;
-      const int32_t seg = wide ? seg_cost : 0;  // what starting a segment in a piece costs
-      auto next_room = [&]() {
-        if (wide) ++wide_slot;
-        room = wide ? next_wide_room() : slot_room;
-      };
-      if (wide && room < seg + min_piece) next_room();  // too little left for a piece worth its set-up
-      int64_t left = tile_tokens;            // tokens of the tile not yet in a piece
-      int64_t segs_left = (int64_t)all.size();  // segments of the tile not yet finished
-      // no tiny last piece: a remainder that would cost less than `small` stays with the piece before it
-      // (small next to a slot's share: the slot that keeps it runs that much longer than the others)
-      const int64_t small = wide ? std::min<int64_t>(min_piece + seg, chain_budget / 8) : min_piece;
-      auto fit_room = [&]() {
-        const int64_t need = left + seg * segs_left;  // room that takes all that is left
-        if (need > room && need - room < small - seg) room = (int32_t)need;
-      };
-      fit_room();
-      std::vector<Link> cur;
-      auto close_piece = [&]() {
-        if (!cur.empty()) emit(b - a, cur, std::vector<int32_t>(rows), -1, wide ? wide_slot : -1);
-        cur.clear();
-      };
-      for (auto l : all) {
-        const bool aligned = align_cuts && !(l.flags & VA_LINK_SLOTS);
-        while (l.tok_begin < l.tok_end) {
-          int32_t take = room > seg ? std::min(room - seg, l.tok_end - l.tok_begin) : 0;
-          if (aligned && take < l.tok_end - l.tok_begin) take = take / 16 * 16;  // l.tok_begin is a multiple of 16: segments start at 0, cuts keep it so
-          if (take <= 0) {  // no room left to start (or go on with) the segment here: the piece ends
-            if (!cur.empty() && left + seg * segs_left < small) {  // ... unless what is left is too little for a piece of its own
-              room = (int32_t)(left + seg * segs_left);
-              continue;
-            }
-            close_piece();
-            next_room();
-            fit_room();
-            continue;
-          }
-          Link piece = l;
-          piece.tok_end = l.tok_begin + take;
-          cur.push_back(piece);
-          l.tok_begin += take;
-          left -= take;
-          room -= take + seg;
-          if (wide) wide_left -= take + seg;
-          if (room <= 0 && left > 0) {
-            if (left + seg * segs_left < small) {  // too little for a piece of its own: it stays with this one
-              room = (int32_t)(left + seg * segs_left);
-              continue;
-            }
-            close_piece();
-            next_room();
-            fit_room();
-          }
-        }
-        --segs_left;
-      }
-      close_piece();
-      if (wide) {
-        if (room <= 0) next_room();
-        wide_room = room;
-      }
+      cut_walk(all, [&](const std::vector<Link>& cur) { emit(b - a, cur, tile_rows(a, b)); });
     }
   }
 
@@ -521,35 +645,40 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     }
     if (units.empty()) continue;
     if (kind == 1 && std::any_of(out.items.begin(), out.items.end(), [](const Item& it) { return it.kind == 1 && it.slot >= 0; })) {
-      // Packed wide pieces: every slot walks the same number of tokens, so the slots simply follow
-      // each other (slot k on die k % 8); wide items outside the packing get slots of their own.
+      // Packed wide pieces: slot id = group * lanes + lane.  Every group costs the same, and its
+      // lanes walk the same tokens at the same pace: group g goes to die g % 8 as a whole, where
+      // the K/V its lanes share is fetched from HBM once and found in that die's L2 by the others.
+      // Wide items outside the packing get slots of their own on the die with the fewest.
       std::vector<std::vector<int32_t>> by_slot;
       for (int32_t i = 0; i < (int32_t)out.items.size(); ++i) {
         const Item& it = out.items[i];
-        if (it.kind != 1) continue;
-        if (it.slot >= 0) {
-          if ((size_t)it.slot >= by_slot.size()) by_slot.resize(it.slot + 1);
-          by_slot[it.slot].push_back(i);
-        }
+        if (it.kind != 1 || it.slot < 0) continue;
+        if ((size_t)it.slot >= by_slot.size()) by_slot.resize(it.slot + 1);
+        by_slot[it.slot].push_back(i);
       }
-      for (int32_t i = 0; i < (int32_t)out.items.size(); ++i)
-        if (out.items[i].kind == 1 && out.items[i].slot < 0) by_slot.push_back({i});
-      by_slot.erase(std::remove_if(by_slot.begin(), by_slot.end(), [](const std::vector<int32_t>& v) { return v.empty(); }),
-                    by_slot.end());
-      // Slots were filled in the order of the tiles, so neighbouring slots walk the same request's
-      // view (the pieces of one chunk's query tiles) at the same pace: they go to ONE die, where the
-      // K/V they share is fetched from HBM once and found in that die's L2 by the others.  Slot k of
-      // the launch runs on die k % 8: die d takes the d-th run of n / 8 consecutive slots.
-      while (by_slot.size() % kXcds) by_slot.emplace_back();  // empty slots
-      const size_t per_die = by_slot.size() / kXcds;
+      std::vector<std::vector<int32_t>> die_slots[kXcds];
+      for (size_t k = 0; k < by_slot.size(); ++k)
+        if (!by_slot[k].empty()) die_slots[(k / lanes) % kXcds].push_back(std::move(by_slot[k]));
+      for (int32_t i = 0; i < (int32_t)out.items.size(); ++i) {
+        if (out.items[i].kind != 1 || out.items[i].slot >= 0) continue;
+        int least = 0;
+        for (int d = 1; d < kXcds; ++d)
+          if (die_slots[d].size() < die_slots[least].size()) least = d;
+        die_slots[least].push_back({i});
+      }
+      size_t per_die = 0;
+      for (int d = 0; d < kXcds; ++d) per_die = std::max(per_die, die_slots[d].size());
+      // slot k of the launch runs on die k % 8 (the kernel maps its workgroups that way)
       out.wide_slots.assign(1, 0);
-      for (size_t k = 0; k < by_slot.size(); ++k) {
-        const auto& members = by_slot[(k % kXcds) * per_die + k / kXcds];
-        for (int32_t m : members) sorted.push_back(out.items[m]);
+      for (size_t k = 0; k < per_die * kXcds; ++k) {
+        const auto& on_die = die_slots[k % kXcds];
+        if (k / kXcds < on_die.size())
+          for (int32_t m : on_die[k / kXcds]) sorted.push_back(out.items[m]);
         out.wide_slots.push_back((int32_t)sorted.size());
       }
       const Item padding{0, 0, 0, -1, 0, 1, -1, -1};
-      while (sorted.size() % kXcds) sorted.push_back(padding);  // outside every slot
+      // (outside every slot; a launch has at least as many items as slots)
+      while (sorted.size() % kXcds || sorted.size() + 1 < out.wide_slots.size()) sorted.push_back(padding);
       out.n_wide = (int32_t)sorted.size();
       continue;
     }
@@ -803,10 +932,12 @@ extern "C" int64_t va_plan_fixed_words(const VaPlanCapacity* cap) {
 //     chunk >= total_tokens / target, plus one for the halved last chunk, so items <= 2 tiles + target
 //     with tiles <= sub-requests; every item carries one link; a query row enters the partial list
 //     once per chunk of its run;
-//   * chains: tiles of up to wide_tile rows (the last one of a chain may be narrow); a tile is
-//     split into round(its tokens / budget) pieces with budget >= all chain tokens / target, so
-//     the extra pieces number at most target and items <= tiles + target per class; a tile has
-//     one link per member plus one per cut; a split tile's rows enter the partial list once per piece.
+//   * chains: tiles of up to wide_tile rows (the last one of a chain may be narrow); a narrow tile
+//     is split into round(its tokens / budget) pieces with budget >= all chain tokens / target; wide
+//     tiles are cut in bundles of `lanes` tiles, at most 7 cuts of at most `lanes` items each with
+//     8 x lanes <= target, and a chain's last bundle may be walked in up to `lanes` parts side by
+//     side; so items <= tiles + chains x lanes + target per class; a tile has one link per member plus
+//     one per cut or part; a split tile's rows enter the partial list once per piece.
 extern "C" int va_plan_capacity(const VaShape* shape, const VaPlanParams* params, const VaPlanLimits* lim,
                                 VaPlanCapacity* capacity) {
   if (!shape || !lim || !capacity) return va_fail(VA_ERR_ARG, "null argument");
@@ -846,15 +977,18 @@ extern "C" int va_plan_capacity(const VaShape* shape, const VaPlanParams* params
   if (chains > 0 && chain_rows > 0) {
     const int64_t tile_rows = wide_tile ? wide_tile : q_tile;
     const int64_t tiles = chain_rows / tile_rows + chains;  // per chain: floor(rows / tile) + 1
+    // the last bundle of a chain may hold fewer tiles than a group has lanes and be walked in parts
+    // side by side: up to `lanes` items, one more link each and `lanes` x tile rows more partial states
+    const int64_t lanes = std::max<int64_t>(1, std::min<int64_t>(target, std::max(1, 256 / shape->num_kv_heads)) / kXcds);
     if (wide_tile) {
-      wide += tiles + target;
+      wide += tiles + chains * lanes + target;
       narrow += chains + target;
     } else {
       narrow += tiles + target;
     }
-    const int64_t chain_items = tiles + target + (wide_tile ? chains + target : 0);
+    const int64_t chain_items = tiles + target + (wide_tile ? chains * (lanes + 1) + target : 0);
     links += tiles * members + chain_items;
-    partials += chain_rows + tile_rows * target;
+    partials += chain_rows + tile_rows * (target + (wide_tile ? chains * lanes : 0));
   }
   links += narrow + wide;
   auto round8 = [](int64_t x) { return (x + 7) / 8 * 8; };

@@ -45,11 +45,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # carried here together with the digest of the kernel sources they were measured on
 # (csrc_digest()), and are reported only while that digest is the one of the sources in the tree.
 MEASURED_TRAFFIC = {
-    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_161_993 + 8_981) + 1024 * (17_894 + 512), "csrc": "a04ae49546c72144"},
-    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_651 + 4_712) + 1024 * (9_302 + 64), "csrc": "a04ae49546c72144"},
-    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_583_551 + 1024 * 131_446, "csrc": "a04ae49546c72144"},
-    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (2_386_998 + 1_628_624 + 25_927) + 1024 * (50_575 + 7_079 + 10_624),
-                              "csrc": "a04ae49546c72144"},
+    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_162_239 + 8_982) + 1024 * (17_893 + 512), "csrc": "b7e68d34c0c87bd0"},
+    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_650 + 4_712) + 1024 * (9_303 + 64), "csrc": "b7e68d34c0c87bd0"},
+    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_563_333 + 1024 * 131_451, "csrc": "b7e68d34c0c87bd0"},
+    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (439_670 + 1_628_612 + 24_373) + 1024 * (47_442 + 7_079 + 10_624),
+                              "csrc": "b7e68d34c0c87bd0"},
 }
 
 

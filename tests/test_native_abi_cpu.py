@@ -318,8 +318,9 @@ def test_compute_entry_points_refuse_cpu_tensors():
 def _packed_slot_loads(chunk_tokens, views, coverage=True):
     """Plan prefill chunks of `chunk_tokens` new tokens, one per entry of `views` (the lengths of the
     context segments of the chunk's view; its own block holds 100 tokens before the chunk), at
-    16 q / 4 kv heads of 256 dims.  Returns (counts, total tokens walked, per-slot loads): a slot's
-    load is the tokens it walks plus the set-up of every (piece, segment) it holds, worth ~640 tokens."""
+    16 q / 4 kv heads of 256 dims.  Returns (counts, total tokens walked, per-slot loads, per-slot walks):
+    a slot's load is the tokens it walks plus the set-up of every (piece, segment) it holds, worth ~640
+    tokens; its walk is the list of (first kv entry, first token, last token) of its links in order."""
     page = 16
     qo, kvp, kvi, lens, flags, chain, sw = [0], [0], [], [], [], [], []
     n_rows = 0
@@ -345,34 +346,51 @@ def _packed_slot_loads(chunk_tokens, views, coverage=True):
     # no piece too small to be worth a set-up of its own: at least ~384 tokens + a segment's 640, unless
     # the slots themselves are so small that a remainder of that size would unbalance them (an eighth of a slot)
     assert min(int(it[4]) + 640 * int(it[1]) for it in items[: slots[-1]]) >= min(384 + 640, sum(loads) // 64 // 8) - 16
-    return counts, int(items[: slots[-1], 4].sum()), loads
+    walks = [[tuple(int(x) for x in l[:3]) for it in items[a:b] for l in links[it[0]: it[0] + it[1]]]
+             for a, b in zip(slots, slots[1:])]
+    return counts, int(items[: slots[-1], 4].sum()), loads, walks
 
 
 def test_few_wide_tiles_are_packed_into_slots_of_equal_length():
     """Prefill chunks whose wide tiles (32 tokens x 4 heads each) cannot fill 64 workgroup slots per
     kv head evenly: views of 1.5k to 30k tokens, and cut one by one into similar pieces the tiles
-    would still fill the slots unevenly.  The planner lays all walks end to end and gives every
-    slot the same share, set-ups included; a slot holds the end of one tile and the start of the
-    next.  The longest slot is the time of the launch (one workgroup per CU, one round): it must
-    stay close to the mean, and no slot may be left to take a long remainder."""
-    # 8 tiles for 64 slots: every tile is cut in about eight
-    counts, total, loads = _packed_slot_loads(64, [(512, 30000), (512, 1500), (512, 12345), (512, 22222)])
+    would still fill the slots unevenly.  The planner bundles the tiles of a chunk (they walk the
+    same view), lays the bundles' walks end to end and gives every group of eight slots -- the
+    slots of one die, which walk a bundle side by side -- the same share, set-ups included; a group
+    holds the end of one bundle and the start of the next.  The longest slot is the time of the
+    launch (one workgroup per CU, one round): it must stay close to the mean, and no slot may be
+    left to take a long remainder."""
+    # 8 tiles for 64 slots: two tiles a chunk, so a bundle walks four quarters of its view side by side.
+    # A group's share is ~3000 tokens here, of which a set-up is a fifth and the least piece a third:
+    # that is the grain the groups can be equal to.
+    counts, total, loads, _ = _packed_slot_loads(64, [(512, 30000), (512, 1500), (512, 12345), (512, 22222)])
     assert total == 2 * (4 * 512 + 30000 + 1500 + 12345 + 22222) + sum(2 * 100 + 32 + 64 for _ in range(4))
     # the longest slot is the time of the launch; slots at the end may be short or empty
-    assert sum(loads) >= 0.92 * 64 * max(loads), (min(loads), max(loads), sum(loads) / 64)
-    # 64 tiles for 64 slots (four chunks of 512 tokens over views of two to five blocks): most slots hold the
-    # end of one tile and the start of the next
+    assert sum(loads) >= 0.84 * 64 * max(loads), (min(loads), max(loads), sum(loads) / 64)
+    # 64 tiles for 64 slots (four chunks of 512 tokens over views of two to five blocks: two bundles of eight
+    # tiles a chunk): most groups hold the end of one bundle and the start of the next
     views = [(512, 9000, 14000), (512, 2500), (512, 7000, 8000, 9000, 6000), (512, 900, 11000, 3000)]
-    counts, total, loads = _packed_slot_loads(512, views, coverage=False)
+    counts, total, loads, walks = _packed_slot_loads(512, views, coverage=False)
     assert total == sum(16 * (sum(v) + 100) + sum(range(32, 513, 32)) for v in views)
     assert sum(loads) >= 0.96 * 64 * max(loads) and min(loads) > 0, (min(loads), max(loads), sum(loads) / 64)
+    # Lockstep: slot k of the launch runs on die k % 8, and the eight slots of a die walk the same tokens
+    # in the same order (one of them fetches a K/V tile from HBM, the others find it in the die's L2).
+    # Only the chunk's own block ends where each tile's causal limit puts it: 32 tokens apart.
+    for die in range(8):
+        lanes = walks[die::8]
+        assert len(lanes) == 8
+        for lane in lanes[1:]:
+            assert len(lane) == len(lanes[0])
+            for (kv, t0, t1), (kv0, u0, u1) in zip(lane, lanes[0]):
+                assert (kv, t0) == (kv0, u0) and 0 <= t1 - u1 <= 7 * 32
 
 
 def test_prefill_tiles_are_cut_by_tokens_on_page_group_boundaries():
     """Two prefill requests of one 32-row tile each, one over 30000 context tokens
     in three segments of odd lengths, one over 700: too few tiles to fill the
     machine, so the planner splits them by tokens.  The long tile must come out
-    in many pieces of similar weight, the short one in at most three; with pages of 16
+    in many pieces (eight parts of its walk side by side on the slots of a die, each cut where a
+    die's share ends) that load the dies alike, the short one in at most three; with pages of 16
     tokens every cut inside a segment lies on a 16-token boundary, with pages of
     4 it need not; every visible pair is covered once either way."""
     for page in (16, 4):
@@ -394,18 +412,21 @@ def test_prefill_tiles_are_cut_by_tokens_on_page_group_boundaries():
         check_coverage(blob, qo, kvp, lens, flags, sw, n_rows)
         h, items, links, *_ = decode_plan(blob)
         real = [it for it in items if it[2] > 0]
-        weight = {}
+        pieces = {}
         for it in real:
             ls = links[it[0]: it[0] + it[1]]
-            # what a piece costs its workgroup: the tokens it walks and ~640 more for every segment it stages
-            tokens = sum(int(l[2] - l[1]) for l in ls) + 640 * len(ls)
             long_one = any(int(l[0]) < kvp[3] for l in ls)  # kv_begin inside the first request's tables
-            weight.setdefault(long_one, []).append(tokens)
-        # (the short tile, 748 tokens in two segments, is worth about two slots' shares with its set-ups:
+            pieces[long_one] = pieces.get(long_one, 0) + 1
+        # (the short tile, 748 tokens in two segments, is worth less than a group's share with its set-ups:
         # it may be cut once or twice, not shredded)
-        assert len(weight[False]) <= 3, "the short tile was cut in many pieces"
-        assert len(weight[True]) >= 20, "the long tile was not cut by its tokens"
-        assert max(weight[True]) <= 1.3 * sorted(weight[True])[1], weight[True]  # (one piece takes what is left)
+        assert pieces[False] <= 3, "the short tile was cut in many pieces"
+        assert pieces[True] >= 20, "the long tile was not cut by its tokens"
+        # What a workgroup slot costs: the tokens it walks and ~640 more for every segment it stages.  The
+        # eight slots of a die walk a tile's eight parts side by side: the dies must come out alike.
+        slots = blob[h[H["OFF_WIDE_SLOTS"]]: h[H["OFF_WIDE_SLOTS"]] + h[H["N_WIDE_SLOTS"]] + 1]
+        loads = [int(items[a:b, 4].sum()) + 640 * int(items[a:b, 1].sum()) for a, b in zip(slots, slots[1:])]
+        dies = [max(loads[d::8]) for d in range(8) if max(loads[d::8]) > 0]
+        assert len(dies) >= 4 and max(dies) <= 1.3 * sum(dies) / len(dies), dies
         inner = [int(l[1]) for it in real for l in links[it[0]: it[0] + it[1]] if l[1] > 0]
         assert inner, "no cut inside a segment"
         if page >= 16:
