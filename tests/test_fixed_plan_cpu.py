@@ -65,6 +65,38 @@ def test_fixed_plans_share_one_header_and_cover_every_pair_once(prefill, kernel,
     assert all(np.array_equal(h, headers[0]) for h in headers)
 
 
+@pytest.mark.parametrize("heads", [(16, 4, 256), (4, 2, 64), (8, 8, 128), (4, 1, 64)])
+def test_capacity_holds_chains_packed_in_bundles(heads):
+    """Prefill chunks of a few wide tiles over views of several thousand tokens: the planner packs
+    their tiles in bundles (the slots of a die walk a bundle's tokens side by side; a chain's last
+    bundle of few tiles is walked in parts), which makes more items, links and partial states than
+    one per tile.  The capacity computed from the limits alone must hold every such plan, and the
+    plan must cover every visible pair once."""
+    rng = random.Random(heads[0] * 100 + heads[1])
+    for case in range(6):
+        page = rng.choice([16, 4])
+        target = rng.choice([0, 0, 8, 64])
+        qo, kvp, kvi, lens, flags, chain, sw = [0], [0], [], [], [], [], []
+        n_rows, n_chains, members = 0, rng.randint(1, 5), 1
+        for r in range(n_chains):
+            new_tokens = rng.choice([1, 9, 33, 64, 65, 138, 300])
+            rows = list(range(n_rows, n_rows + new_tokens))
+            n_rows += new_tokens
+            context = [rng.choice([5, 100, 700, 1500, 4000]) for _ in range(rng.randint(0, 3))]
+            members = max(members, len(context) + 1)
+            for length in context + [rng.choice([0, 7, 100]) + new_tokens]:
+                kvi += list(range(len(kvi), len(kvi) + -(-length // page)))
+                kvp.append(len(kvi)); lens.append(length); chain.append(r)
+                flags.append(0)
+                sw += rows; qo.append(len(sw))
+            flags[-1] = 1  # the chunk's own block is the causal one
+        limits = native.VaPlanLimits(0, 0, n_chains, members, n_rows, n_rows)
+        rc, blob, counts, cap = fixed_plan((qo, kvp, kvi, lens, flags, chain, sw, n_rows), limits, heads=heads, page=page,
+                                           dtype=native.VA_BF16, kernel=native.VA_KERNEL_MFMA, target=target)
+        assert rc == 0, (case, native.lib.va_last_error())
+        check_coverage(blob, qo, kvp, lens, flags, sw, n_rows, fixed=True)
+
+
 def test_padding_per_die_never_exceeds_a_capacity_the_real_items_fit():
     """One heavy unit and many light ones: dealing by load alone gives one die few
     entries and the others many, and padding every die to the longest list would
