@@ -318,18 +318,18 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   // Chains.  When the tiles of all chains are many (several rounds of one workgroup per CU) every
   // tile is one work item and the hardware hands them out as CUs fall free.  When they are few --
   // a handful of prefill chunks in a continuous batch, whose views differ in length by a factor
-  // of thirty -- whole tiles cannot fill the machine evenly, so the walk of all tiles, laid end to
-  // end, is cut into equal token budgets instead: one budget per workgroup ("slot") of a launch of
-  // one workgroup per CU.  A slot runs its pieces one after the other; a tile cut in pieces yields
-  // partial states that the merge kernel folds.  Every slot then walks the same number of tokens
-  // (the cost of a wide tile is its tokens: all its rows share each K/V tile) and the launch is
-  // one even round, where 2.25 rounds of uneven items used to take the time of three.
-  // Narrow tiles of chains (the last rows of a request) are cut by the same budget, one item a piece.
+  // of thirty -- whole tiles cannot fill the machine evenly, so the walks of the wide tiles, laid end
+  // to end, are cut into equal budgets instead, for a launch of one workgroup ("slot") per CU.  A slot
+  // runs its pieces one after the other; a tile cut in pieces yields partial states that the merge
+  // kernel folds.  Every slot then costs the same (the cost of a wide tile is its tokens, all its rows
+  // share each K/V tile, plus a set-up per segment) and the launch is one even round, where 2.25
+  // rounds of uneven items used to take the time of three.
+  // Narrow tiles of chains (the last rows of a request) are cut by a token budget, one item a piece.
   const int64_t slots_wanted = std::max(1, 256 / shape->num_kv_heads);
   int64_t chain_budget = INT64_MAX;
   // A piece of a wide tile stages its query tile once per segment of the view it walks (the query is
   // rotated for every block anew), which costs about as much as walking `seg_cost` tokens: the packing
-  // charges every (piece, segment) to the slot's room.  A tile's remainder that would cost less than
+  // charges every (piece, segment) to the room it fills.  A remainder that would cost less than
   // `min_piece` stays with the piece before it.
   const int32_t seg_cost = 10 * gran;
   const int32_t min_piece = 6 * gran;
