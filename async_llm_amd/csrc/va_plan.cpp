@@ -230,7 +230,9 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
       if (tl.second - tl.first > q_tile) wide_chain_tokens += walked;
     }
   }
-  total_tokens += chain_tokens;
+  // (the chunk cuts the runs of stand-alone sub-requests only -- chains are cut by budgets of their own,
+  // below -- so it is sized from their tokens alone: in a mixed batch the prefill chunks' long walks
+  // would otherwise triple it, and the decode items would run in two long rounds instead of four short ones)
   int32_t kv_chunk = params && params->kv_chunk > 0 ? round_up(params->kv_chunk, gran) : 0;
   if (kv_chunk == 0) {
     const int64_t per_item = (total_tokens + target - 1) / target;

@@ -2,6 +2,8 @@
 // the partial-state merge kernel.  The matrix-core kernels live in va_mfma_stream.hip and va_mfma_wide.hip.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -430,8 +432,9 @@ __global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
 // merge of partial states: one workgroup of kMergeWaves waves per (row, q head)
 // ---------------------------------------------------------------------------
 // The launch is short and made of dependent loads (row list -> partial states), so it is laid out
-// for latency: wave w folds partials w, w + kMergeWaves, ... of the row, eight per round with all
-// their loads in flight together, and the running states meet in LDS.  Lane l owns dims l, l + 64, ...
+// for latency: wave w folds partials w, w + kMergeWaves, ... of the row, eight per round (the last
+// round exactly what is left) with all their loads in flight together, and the running states meet
+// in LDS.  Lane l owns dims l, l + 64, ...
 // Four waves for a decode batch (few rows, up to dozens of partial states each); one wave when the
 // rows are many (split prefill tiles: thousands of rows of a few states each), where four times as
 // many rows in flight per CU count for more than the parallel fold.
@@ -453,15 +456,15 @@ __global__ __launch_bounds__(64 * kMergeWaves) void merge_kernel(MergeArgs a) {
   const int n_d = (a.head_dim + 63) / 64;  // dims per lane: d = lane + 64*k (at most 4 for D = 256)
   float mm = kNegBig, ll = 0.f;
   float av[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int i0 = b + wave; i0 < e; i0 += 8 * kMergeWaves) {
-    float mp[8], lp[8], ap[8][4];
+  // fold partials i0, i0 + kMergeWaves, ... (n of them): all loads first, then the fold in order
+  auto fold = [&](int i0, auto n_tag) __attribute__((always_inline)) {
+    constexpr int n = decltype(n_tag)::value;
+    float mp[n], lp[n], ap[n][4];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int iu = i0 + u * kMergeWaves;
-      const int i = min(iu, e - 1);
-      const long long slot = (long long)a.row_ids[i] * a.num_q_heads + hq;
-      mp[u] = iu < e ? a.part_ml[slot * 2] : kNegBig;
-      lp[u] = iu < e ? a.part_ml[slot * 2 + 1] : 0.f;
+    for (int u = 0; u < n; ++u) {
+      const long long slot = (long long)a.row_ids[i0 + u * kMergeWaves] * a.num_q_heads + hq;
+      mp[u] = a.part_ml[slot * 2];
+      lp[u] = a.part_ml[slot * 2 + 1];
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const int d = lane + 64 * k;
@@ -469,7 +472,7 @@ __global__ __launch_bounds__(64 * kMergeWaves) void merge_kernel(MergeArgs a) {
       }
     }
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < n; ++u) {
       const float m_new = fmaxf(mm, mp[u]);
       const float sa = exp2f(mm - m_new), sb = exp2f(mp[u] - m_new);
       ll = ll * sa + lp[u] * sb;
@@ -477,7 +480,21 @@ __global__ __launch_bounds__(64 * kMergeWaves) void merge_kernel(MergeArgs a) {
       for (int k = 0; k < 4; ++k) av[k] = av[k] * sa + ap[u][k] * sb;
       mm = m_new;
     }
+  };
+  // this wave's partials, eight per round; the last round takes exactly what is left (a split
+  // prefill row has two or three states: a padded round of eight would quadruple its loads)
+  int i0 = b + wave;
+  int mine = i0 < e ? (e - i0 + kMergeWaves - 1) / kMergeWaves : 0;
+  for (; mine >= 8; mine -= 8, i0 += 8 * kMergeWaves) fold(i0, std::integral_constant<int, 8>{});
+  if (mine & 4) {
+    fold(i0, std::integral_constant<int, 4>{});
+    i0 += 4 * kMergeWaves;
   }
+  if (mine & 2) {
+    fold(i0, std::integral_constant<int, 2>{});
+    i0 += 2 * kMergeWaves;
+  }
+  if (mine & 1) fold(i0, std::integral_constant<int, 1>{});
   if constexpr (kMergeWaves > 1) {
     // fold the waves' states: wave 0 collects
     __shared__ float s_ml[kMergeWaves][2];

@@ -45,11 +45,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # carried here together with the digest of the kernel sources they were measured on
 # (csrc_digest()), and are reported only while that digest is the one of the sources in the tree.
 MEASURED_TRAFFIC = {
-    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_161_951 + 8_982) + 1024 * (17_896 + 512), "csrc": "4970917e49a89f10"},
-    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_648 + 4_712) + 1024 * (9_303 + 64), "csrc": "4970917e49a89f10"},
-    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_587_673 + 1024 * 131_414, "csrc": "4970917e49a89f10"},
-    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (439_790 + 1_628_824 + 24_373) + 1024 * (47_436 + 7_080 + 10_624),
-                              "csrc": "4970917e49a89f10"},
+    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_162_131 + 8_988) + 1024 * (17_894 + 512), "csrc": "0535ec7c1795becd"},
+    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_655 + 4_723) + 1024 * (9_303 + 64), "csrc": "0535ec7c1795becd"},
+    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_582_743 + 1024 * 131_429, "csrc": "0535ec7c1795becd"},
+    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (439_575 + 1_625_692 + 27_057) + 1024 * (47_437 + 12_409 + 10_624),
+                              "csrc": "0535ec7c1795becd"},
 }
 
 
