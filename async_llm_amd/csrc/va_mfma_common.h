@@ -191,10 +191,10 @@ struct TableQueryUnit {
         const S xb = __builtin_bit_cast(S, (uint16_t)(wb[w] >> (16 * b)));
         const float sn = p.t < 0 ? -st[2 * w + b] : st[2 * w + b];
         // the table mode's arithmetic of rope_pair: fp32, one rounding at the end
-        y1[b] = round_through<E>(mul_rounded(ct[2 * w + b], E::load(xa)) - mul_rounded(sn, E::load(xb)));
-        y2[b] = round_through<E>(mul_rounded(ct[2 * w + b], E::load(xb)) + mul_rounded(sn, E::load(xa)));
+        y1[b] = mul_rounded(ct[2 * w + b], E::load(xa)) - mul_rounded(sn, E::load(xb));
+        y2[b] = mul_rounded(ct[2 * w + b], E::load(xb)) + mul_rounded(sn, E::load(xa));
       }
-      lo[w] = Mma<E>::pack(y1[0], y1[1]);  // already representable: the conversions are exact
+      lo[w] = Mma<E>::pack(y1[0], y1[1]);  // the one rounding (to nearest even, as E::store rounds)
       hi[w] = Mma<E>::pack(y2[0], y2[1]);
     }
     o0 = make_uint4(lo[0], lo[1], lo[2], lo[3]);

@@ -286,7 +286,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         // -> query pieces and cos|sin entries) is paid once per batch, not once per row (row by row
         // this set-up was an eighth of the kernel on long views of many blocks).
         constexpr int kUnits = kChunks / 2, kRowStep = kWideThreads / kUnits, kIts = 128 / kRowStep;
-        constexpr int kBatch = kIts < 2 ? kIts : 2;
+        constexpr int kBatch = kIts < 4 ? kIts : 4;
         static_assert(kWideThreads % kUnits == 0 && 128 % kRowStep == 0 && kIts % kBatch == 0, "staging pattern");
         const int x = tid % kUnits, rl0 = tid / kUnits;
         const int pair_units = a.rope.rotary_dim / 16;
