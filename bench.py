@@ -45,11 +45,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # carried here together with the digest of the kernel sources they were measured on
 # (csrc_digest()), and are reported only while that digest is the one of the sources in the tree.
 MEASURED_TRAFFIC = {
-    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_162_131 + 8_988) + 1024 * (17_894 + 512), "csrc": "0535ec7c1795becd"},
-    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_655 + 4_723) + 1024 * (9_303 + 64), "csrc": "0535ec7c1795becd"},
-    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_582_743 + 1024 * 131_429, "csrc": "0535ec7c1795becd"},
-    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (439_575 + 1_625_692 + 27_057) + 1024 * (47_437 + 12_409 + 10_624),
-                              "csrc": "0535ec7c1795becd"},
+    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_161_327 + 8_988) + 1024 * (17_895 + 512), "csrc": "641d34d174eb822f"},
+    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_575 + 4_715) + 1024 * (9_303 + 64), "csrc": "641d34d174eb822f"},
+    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_674_513 + 1024 * 131_521, "csrc": "641d34d174eb822f"},
+    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (440_165 + 1_625_516 + 27_058) + 1024 * (47_439 + 12_409 + 10_624),
+                              "csrc": "641d34d174eb822f"},
 }
 
 
