@@ -67,6 +67,16 @@ __device__ __forceinline__ int swz(int r) {
 }
 
 
+// max over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (the contraction groups of an MFMA row) with the two
+// row-swapping instructions of gfx950, no trip through the LDS crossbar: with both operands x,
+// v_permlane16_swap leaves (rows 0 0 2 2, rows 1 1 3 3) of x and v_permlane32_swap (low low, high high).
+__device__ __forceinline__ float max_over_contraction_groups(float x) {
+  const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
 template <typename E, int kD>
 __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void attn_stream_kernel(AttnArgs a) {
   using S = typename E::storage;
@@ -238,20 +248,28 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
         ring_barrier<0>();
       }
 
-      // the page of the tile requested at the end of this iteration: looked up now, so the lookup's
-      // latency is covered by the computation
       const bool refill = i + kBuffers < n_tiles;
-      const int next_page = (decltype(uniform_tag)::value && refill) ? page_of(i + kBuffers) : 0;
+      int next_page = 0;
       const int t0 = tok_begin + i * kStreamTok;
       const char* kt = lds + (i % kBuffers) * kBufferBytes;
       const char* vt = kt + kTileUnits * 16;
       if (pv_wave) {
         // scores: S^T = K . Q^T; lane (j, kg) supplies dims [32s + 8kg, +8) of token t0 + j
+        // every K fragment is requested before the first product (left to itself the compiler reads
+        // them one by one into one set of registers: an LDS latency per product)
+        va_u32x4 kfr[kSteps];
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) kfr[s] = *(const va_u32x4*)(kt + k_byte[s % 4] + 256 * (s / 4));
+        __builtin_amdgcn_sched_barrier(0);
         va_f32x4 sc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s = 0; s < kSteps; ++s)
-          sc = Mma<E>::run(*(const va_u32x4*)(kt + k_byte[s % 4] + 256 * (s / 4)), qf[s], sc);
+        for (int s = 0; s < kSteps; ++s) sc = Mma<E>::run(kfr[s], qf[s], sc);
 
+        // The page of the tile requested at the end of this iteration is looked up here: the softmax and
+        // the products below cover the latency -- and not before the score products, because a scalar
+        // load in flight shares its counter with the LDS reads, which then could only be waited for
+        // all at once (every K fragment read a full LDS latency of its own).
+        if (decltype(uniform_tag)::value && refill) next_page = page_of(i + kBuffers);
         // online softmax: this lane holds tokens t0 + 4kg + r of row j
         float tile_max = -INFINITY;
 #pragma unroll
@@ -260,15 +278,15 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
           sc[r] = v;
           tile_max = fmaxf(tile_max, v);
         }
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+        tile_max = max_over_contraction_groups(tile_max);
         const float m_new = fmaxf(m_run, tile_max);
-        const float alpha = exp2f(m_run - m_new);
+        // (the bare instruction: results below 2^-126 become 0 instead of denormal)
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         m_run = m_new;
         float pr[4], psum = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          pr[r] = exp2f(sc[r] - m_new);
+          pr[r] = __builtin_amdgcn_exp2f(sc[r] - m_new);
           psum += pr[r];
         }
         l_run = l_run * alpha + psum;
@@ -297,6 +315,9 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
                                __builtin_amdgcn_perm(vraw[3][w], vraw[2][w], sel)};
           o[t] = Mma<E>::run16(vf, pf, o[t]);
         }
+      }
+      else if (decltype(uniform_tag)::value && refill) {
+        next_page = page_of(i + kBuffers);  // (waves that only load, at head_dim 64)
       }
       // refill this tile's buffer once every wave has consumed it
       if (refill) {
