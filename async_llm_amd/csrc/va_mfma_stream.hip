@@ -87,7 +87,23 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
   extern __shared__ va_u32x4 ring[];  // buffer b: K tile at ring + 2b * kTileUnits, V tile kTileUnits further
 
   const ItemHead where = item_and_head(blockIdx.x, a.num_kv_heads);
-  const int32_t* item = a.items + (long long)where.item * VA_ITEM_WORDS;
+  // The whole item (its first link travels in it) in ONE round of scalar loads: fetched word by word
+  // where each was first needed, the item cost three dependent trips to memory before the first tile
+  // could be requested.
+  typedef int va_i32x4 __attribute__((ext_vector_type(4)));
+  int item[VA_ITEM_WORDS];
+  {
+    const __attribute__((address_space(4))) va_i32x4* words =
+        (const __attribute__((address_space(4))) va_i32x4*)(a.items + (long long)where.item * VA_ITEM_WORDS);
+#pragma unroll
+    for (int w = 0; w < VA_ITEM_WORDS / 4; ++w) {
+      const va_i32x4 x = words[w];
+      item[4 * w + 0] = x[0];
+      item[4 * w + 1] = x[1];
+      item[4 * w + 2] = x[2];
+      item[4 * w + 3] = x[3];
+    }
+  }
   const int hk = where.head;
   const int G = a.num_q_heads / a.num_kv_heads;
   const int n_q = item[VA_I_N_Q];
@@ -138,7 +154,22 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
 
   for (int li = 0; li < item[VA_I_N_LINKS]; ++li) {
     // the first link travels with the item
-    const int32_t* link = li == 0 ? item + VA_I_LINK0 : a.links + (long long)(item[VA_I_LINK_BEGIN] + li) * VA_LINK_WORDS;
+    int link[VA_LINK_WORDS];
+    if (li == 0) {
+#pragma unroll
+      for (int w = 0; w < VA_LINK_WORDS; ++w) link[w] = item[VA_I_LINK0 + w];
+    } else {
+      const __attribute__((address_space(4))) va_i32x4* words = (const __attribute__((address_space(4))) va_i32x4*)(
+          a.links + (long long)(item[VA_I_LINK_BEGIN] + li) * VA_LINK_WORDS);
+#pragma unroll
+      for (int w = 0; w < VA_LINK_WORDS / 4; ++w) {
+        const va_i32x4 x = words[w];
+        link[4 * w + 0] = x[0];
+        link[4 * w + 1] = x[1];
+        link[4 * w + 2] = x[2];
+        link[4 * w + 3] = x[3];
+      }
+    }
     const int lflags = link[VA_L_FLAGS];
     const int qref = link[VA_L_QREF];
     const int kv_begin = link[VA_L_KV_BEGIN];
@@ -343,10 +374,9 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     const int hq = hk * G + g;
     const int d0 = wave * Sh::kDimsPerWave + 4 * kRun * kg;
     if (part_base < 0) {
-      const int32_t* link0 = item + VA_I_LINK0;
-      const long long out_row = (link0[VA_L_FLAGS] & VA_LINK_INDIRECT)
-                                    ? (long long)a.qref_rows[link0[VA_L_QREF] + row_iq]
-                                    : a.sub_worker[link0[VA_L_QREF] + row_iq];
+      const int qref0 = item[VA_I_LINK0 + VA_L_QREF];
+      const long long out_row = (item[VA_I_LINK0 + VA_L_FLAGS] & VA_LINK_INDIRECT) ? (long long)a.qref_rows[qref0 + row_iq]
+                                                                                   : a.sub_worker[qref0 + row_iq];
       S* orow = (S*)a.out + (out_row * a.num_q_heads + hq) * (long long)kD + d0;
       const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
       uint32_t w[2 * kRun];

@@ -45,11 +45,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # carried here together with the digest of the kernel sources they were measured on
 # (csrc_digest()), and are reported only while that digest is the one of the sources in the tree.
 MEASURED_TRAFFIC = {
-    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_164_474 + 8_988) + 1024 * (17_897 + 512), "csrc": "8ebbd31b3b61d37c"},
-    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_596 + 4_715) + 1024 * (9_303 + 64), "csrc": "8ebbd31b3b61d37c"},
-    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_675_835 + 1024 * 131_494, "csrc": "8ebbd31b3b61d37c"},
-    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (440_287 + 1_625_580 + 27_058) + 1024 * (47_445 + 12_410 + 10_624),
-                              "csrc": "8ebbd31b3b61d37c"},
+    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_164_850 + 8_988) + 1024 * (17_900 + 512), "csrc": "1cf17c94a6b28696"},
+    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_099_479 + 4_715) + 1024 * (9_304 + 64), "csrc": "1cf17c94a6b28696"},
+    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_654_373 + 1024 * 131_485, "csrc": "1cf17c94a6b28696"},
+    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (440_246 + 1_625_414 + 27_059) + 1024 * (47_446 + 12_410 + 10_624),
+                              "csrc": "1cf17c94a6b28696"},
 }
 
 
