@@ -11,6 +11,7 @@ the x86 pass, which ignores it with a warning.  Sources compile in parallel.
 
 from __future__ import annotations
 
+import hashlib
 import os
 import subprocess
 import sys
@@ -62,8 +63,15 @@ def build(verbose: bool = True, out: str = LIB_PATH, extra_flags=(), incremental
     """Compile every source and link ``out``.  ``incremental`` keeps objects that are newer than
     their source and every header (same flags assumed); the default recompiles everything."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    tag = "" if out == LIB_PATH and not extra_flags else "." + str(abs(hash((out, tuple(extra_flags)))) % 10 ** 8)
     os.makedirs(OBJ_DIR, exist_ok=True)
+    # objects are named after everything that shapes them besides the source text: the output they
+    # are linked into and every flag (a digest that is the same in every process, unlike hash())
+    flags = repr((out, tuple(extra_flags), COMMON_FLAGS, DEVICE_FLAGS, HOST_FLAGS, sorted(SOURCE_DEVICE_FLAGS.items())))
+    default = out == LIB_PATH and not extra_flags
+    tag = "" if default else "." + hashlib.sha1(flags.encode()).hexdigest()[:10]
+    stamp = os.path.join(OBJ_DIR, "flags" + tag + ".txt")
+    if incremental and not (os.path.exists(stamp) and open(stamp).read() == flags):
+        incremental = False  # the flags changed since these objects were made
     jobs, objects = [], []
     headers = _newest_header() if incremental else 0.0
     for src in HIP_SOURCES + HOST_SOURCES:
@@ -77,6 +85,8 @@ def build(verbose: bool = True, out: str = LIB_PATH, extra_flags=(), incremental
         for f in [pool.submit(_compile_one, hipcc, s, o, list(extra_flags), verbose) for s, o in jobs]:
             f.result()
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-o", out], verbose)
+    with open(stamp, "w") as f:
+        f.write(flags)
     return out
 
 

@@ -34,8 +34,12 @@ int launch_mfma(const AttnArgs& a_in, int dtype, int n_items, int n_wide, int n_
     return va_fail(VA_ERR_ARG, "matrix-core path does not support this dtype/head_dim/group size");
   if (q_tile * g > 16) return va_fail(VA_ERR_ARG, "plan tile of %d rows x %d heads exceeds 16 MFMA rows", q_tile, g);
   if (a.rope.rotary_dim % 16) return va_fail(VA_ERR_ARG, "matrix-core path needs rotary_dim to be a multiple of 16");
-  if (a.q_row_stride % 8 || a.pool_row_stride % 8)
+  if (a.q_row_stride % 8 || a.pool_row_stride % 8 || (uintptr_t)a.q % 16 || (uintptr_t)a.k_pool % 16 ||
+      (uintptr_t)a.v_pool % 16)
     return va_fail(VA_ERR_ARG, "matrix-core path needs 16-byte aligned rows");
+  // the query staging reads the cos|sin entries of a unit in 16-byte loads
+  if (a.rope.mode == VA_ROPE_TABLE && a.rope.rotary_dim > 0 && (uintptr_t)a.rope.cos_sin % 16)
+    return va_fail(VA_ERR_ARG, "matrix-core path needs a 16-byte aligned cos|sin table");
   // the streaming kernel addresses a tile's rows with 32-bit byte offsets from its first row
   if (a.pool_row_stride * 2 * 16 > 0x7fffffffLL) return va_fail(VA_ERR_ARG, "pool rows too far apart");
   if (n_wide > 0 && n_wide_slots > 0) {

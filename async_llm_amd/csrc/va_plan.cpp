@@ -336,10 +336,15 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   const int32_t seg_cost = 10 * gran;
   const int32_t min_piece = 6 * gran;
   if (chain_tiles > 0 && chain_tiles < 4 * slots_wanted) {
-    // (at most `want` <= target cuts are made, which is what bounds a fixed-capacity plan)
+    // The budget cuts the walks of the NARROW chain tiles only (wide tiles are packed in bundles by
+    // budgets of their own, below), so it is their tokens that size it: a narrow tile of t tokens
+    // yields at most t / budget + 1 pieces, all narrow tiles together at most `want` <= target more
+    // pieces than there are tiles -- which is the bound a fixed-capacity plan relies on.  (Sized from
+    // the wide tiles' tokens, a one-row chunk over a long view beside a short wide chunk was cut
+    // into hundreds of pieces.)
     const int64_t want = std::max<int64_t>(1, std::min<int64_t>(target, slots_wanted));
-    const int64_t shared = wide_chain_tokens > 0 ? wide_chain_tokens : chain_tokens;
-    chain_budget = std::max<int64_t>((shared + want - 1) / want, 16 * gran);
+    const int64_t narrow_chain_tokens = chain_tokens - wide_chain_tokens;
+    chain_budget = std::max<int64_t>((narrow_chain_tokens + want - 1) / want, 16 * gran);
   }
   // cuts inside a segment keep to multiples of 16 tokens where the kernels profit (pages of 16
   // tokens or more: a piece that starts on such a boundary is fetched with uniform loads)
@@ -904,6 +909,17 @@ static int write_plan(const Built& b, const VaSubRequests* subs, const VaShape* 
   std::copy(b.row_flags.begin(), b.row_flags.end(), plan_host + off);
   for (int32_t r = subs->n_rows; r < cap_rows; ++r) plan_host[off + r] = VA_ROW_EMPTY;
   off += cap_rows;
+  // The waves of a merge workgroup split a row's states, so rows of many states (long views cut
+  // into many chunks) get more waves; when the rows are many (split prefill tiles: thousands of
+  // rows of a few states each) one wave per row keeps more rows in flight.  A fixed plan decides
+  // from its capacity, a packed one from its counts: either way the word is part of the header the
+  // launches are derived from.  Measured on one MI355X: 17 states per row take 9.9 / 14.7 / 20.6 us
+  // with 4 / 8 / 16 waves, 72 per row 16.4 / 12.0 / 9.5 us.
+  {
+    const int64_t rows = std::max<int64_t>(1, cap ? cap_rows : subs->n_rows);
+    const int64_t per_row = (cap ? cap_row_parts : c.n_row_parts) / rows;
+    h[VA_H_MERGE_WAVES] = rows * shape->num_q_heads >= 8192 ? 1 : per_row >= 48 ? 16 : per_row >= 28 ? 8 : 4;
+  }
   h[VA_H_N_WIDE_SLOTS] = c.n_wide_slots;
   h[VA_H_OFF_WIDE_SLOTS] = off;
   std::copy(b.wide_slots.begin(), b.wide_slots.end(), plan_host + off);

@@ -38,6 +38,7 @@ enum {
   VA_H_OFF_QREF_ROWS,  // parallel to qrefs: the query/output row of each entry (sub_worker[qrefs[k]])
   VA_H_N_WIDE_SLOTS,   // workgroups per kv head of the wide launch (a multiple of 8)
   VA_H_OFF_WIDE_SLOTS, // [n_wide_slots + 1]: slot s runs the wide items [indptr[s], indptr[s + 1]) one after the other
+  VA_H_MERGE_WAVES,    // waves per (row, q head) workgroup of the merge launch: 1, 4, 8 or 16
 };
 
 // item word indices

@@ -555,21 +555,25 @@ int launch_generic(const AttnArgs& a, int n_items, hipStream_t stream) {
   return check_hip(hipGetLastError(), "attention launch");
 }
 
-// `n_row_parts`: partial states over all rows.  The waves of a workgroup split a row's states, so
-// rows of many states (long views cut into many chunks) get more waves: measured on one MI355X,
-// 17 states per row take 9.9 / 14.7 / 20.6 us with 4 / 8 / 16 waves, 72 per row 16.4 / 12.0 / 9.5 us.
+// `waves`: waves per (row, q head) workgroup, chosen by the planner (plan header).
 template <typename E>
-int launch_merge(const MergeArgs& a, int n_rows, int n_row_parts, hipStream_t stream) {
+int launch_merge(const MergeArgs& a, int n_rows, int waves, hipStream_t stream) {
   const dim3 grid((unsigned)n_rows, (unsigned)a.num_q_heads);
-  const int per_row = n_row_parts / (n_rows > 0 ? n_rows : 1);
-  if ((int64_t)n_rows * a.num_q_heads >= 8192) {
-    hipLaunchKernelGGL((merge_kernel<E, 1>), grid, dim3(64), 0, stream, a);
-  } else if (per_row >= 48) {
-    hipLaunchKernelGGL((merge_kernel<E, 16>), grid, dim3(1024), 0, stream, a);
-  } else if (per_row >= 28) {
-    hipLaunchKernelGGL((merge_kernel<E, 8>), grid, dim3(512), 0, stream, a);
-  } else {
-    hipLaunchKernelGGL((merge_kernel<E, 4>), grid, dim3(256), 0, stream, a);
+  switch (waves) {
+    case 1:
+      hipLaunchKernelGGL((merge_kernel<E, 1>), grid, dim3(64), 0, stream, a);
+      break;
+    case 4:
+      hipLaunchKernelGGL((merge_kernel<E, 4>), grid, dim3(256), 0, stream, a);
+      break;
+    case 8:
+      hipLaunchKernelGGL((merge_kernel<E, 8>), grid, dim3(512), 0, stream, a);
+      break;
+    case 16:
+      hipLaunchKernelGGL((merge_kernel<E, 16>), grid, dim3(1024), 0, stream, a);
+      break;
+    default:
+      return va_fail(VA_ERR_ARG, "plan header: %d merge waves (1, 4, 8 or 16)", waves);
   }
   return check_hip(hipGetLastError(), "merge launch");
 }
@@ -704,10 +708,7 @@ static int attention_launches(const void* q_dev, int64_t q_row_stride, const voi
     m.lse_base2 = lse_base2;
     m.num_q_heads = shape->num_q_heads;
     m.head_dim = shape->head_dim;
-    // (a fixed-capacity plan's header holds upper bounds, not counts -- its KV chunk word reads 0 --
-    // and its launches must not depend on the plan: it takes the merge for rows of few states)
-    const int n_row_parts = h[VA_H_KV_CHUNK] == 0 ? 0 : h[VA_H_N_ROW_PARTS];
-    VA_DISPATCH_DTYPE(shape->dtype, rc = va::launch_merge<E>(m, n_rows, n_row_parts, s));
+    VA_DISPATCH_DTYPE(shape->dtype, rc = va::launch_merge<E>(m, n_rows, h[VA_H_MERGE_WAVES], s));
   }
   return rc;
 }

@@ -241,8 +241,14 @@ class SharedCacheAttention:
         return self._workspace
 
     def prepare_workspace(self, profiles) -> None:
-        """Reserve the scratch of every fixed-capacity profile once, before any
-        capture (reference ``attention.py:212-239``)."""
+        """Reserve the scratch of the whole catalogue of fixed-capacity profiles once, before any
+        capture (reference ``attention.py:212-239``).  A profile's ``workspace_requirements()``
+        lists ``(consumer, float_bytes, int_bytes)`` entries: every consumer shares one arena of
+        the largest ``float_bytes`` (here: the partial softmax states of a launch) and owns
+        ``int_bytes`` of table storage of its own, both handed over through
+        ``consumer.reset_workspace_buffer(arena, ints)``.  Everything is allocated before the
+        first consumer is rebound, so an allocation that fails leaves the op and every consumer
+        as they were, not prepared."""
         profiles = tuple(profiles)
         if not profiles:
             return
@@ -250,10 +256,16 @@ class SharedCacheAttention:
             raise RuntimeError("Attention workspace must be prepared once before capture")
         if any(p.attention is not self for p in profiles):
             raise ValueError("Attention workspace profiles must belong to this instance")
-        need = max(int(r) for p in profiles for r in p.workspace_requirements())
-        current = 0 if self._workspace is None else self._workspace.numel()
-        if need > current:
-            self._workspace = torch.empty(need, dtype=torch.uint8, device=self.device)
+        wanted = [entry for p in profiles for entry in p.workspace_requirements()]
+        arena = self._workspace
+        size = max([0 if arena is None else arena.numel()] + [int(float_bytes) for _, float_bytes, _ in wanted])
+        if arena is None or size > arena.numel():
+            arena = torch.empty(size, dtype=torch.uint8, device=self.device)
+        tables = [torch.empty(max(16, int(int_bytes)), dtype=torch.uint8, device=self.device)
+                  for _, _, int_bytes in wanted]
+        for (consumer, _, _), ints in zip(wanted, tables):
+            consumer.reset_workspace_buffer(arena, ints)
+        self._workspace = arena
         self._workspace_prepared = True
 
     # ------------------------------------------------------------------

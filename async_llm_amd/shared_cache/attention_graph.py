@@ -58,10 +58,20 @@ class _FixedPlanBuffers:
         self.counts = native.VaPlanCounts()
         self.header: Optional[np.ndarray] = None
         self.refs: list = []
+        self._arena: Optional[torch.Tensor] = None  # the catalogue's shared scratch, once prepare_workspace ran
+        self._ints: Optional[torch.Tensor] = None
 
-    def workspace_requirements(self) -> List[int]:
-        """Scratch bytes of the launch at capacity; the same for every plan."""
-        return [int(self.counts.workspace_bytes)]
+    def workspace_requirements(self) -> List[tuple]:
+        """``[(consumer, float_bytes, int_bytes)]`` as the reference's profiles report them
+        (``attention_graph.py:62-72, 176-187``): the scratch of the launch at capacity (the same
+        for every plan) and no table storage beyond what the buffers already own."""
+        return [(self, int(self.counts.workspace_bytes), 0)]
+
+    def reset_workspace_buffer(self, arena: torch.Tensor, ints: torch.Tensor) -> None:
+        """Take the arena ``prepare_workspace`` reserved for the whole catalogue."""
+        self._arena, self._ints = arena, ints
+        if self.header is not None and getattr(self, "meta", None) is not None and self.meta.launch is not None:
+            self.meta.launch = self._launch()
 
     def _wait_for_staging(self) -> None:
         # the pinned staging tensors are reused: the previous plan's copies must have left them
@@ -96,9 +106,11 @@ class _FixedPlanBuffers:
     def _launch(self):
         from .attention import LaunchPlan
 
-        need = self.workspace_requirements()[0]
-        return LaunchPlan(self.header, self.blob, self.kv_indices, self.counts,
-                          self.attention._ensure_workspace(need))
+        need = int(self.counts.workspace_bytes)
+        arena = self._arena
+        if arena is None or arena.numel() < need:
+            arena = self.attention._ensure_workspace(need)
+        return LaunchPlan(self.header, self.blob, self.kv_indices, self.counts, arena)
 
 
 class SharedDecodeAttentionBuffers(_FixedPlanBuffers):

@@ -26,6 +26,7 @@ import torch
 
 from .kvcache import MHAKVCache
 from .shared_cache import CacheBlock, PrefillSpec, SharedCacheAttention, WorkerGroup
+from .shared_cache.mrope import get_rope_index
 from .shared_cache.session_planning import plan_decode_writes
 
 
@@ -210,7 +211,13 @@ def mrope_decode(device, workers: int = 8, blocks_per_view: int = 8, block_len: 
     rd, section = 128 if D >= 128 else D, (24, 20, 20) if D >= 128 else (D // 2 - 2 * (D // 8), D // 8, D // 8)
     side = int(round(image_tokens ** 0.5))
     assert side * side == image_tokens
-    span = block_len - image_tokens + side
+    # a block's tokens: text, one image of side x side merged patches (grid 1 x 2 side x 2 side at
+    # merge size 2), text; its span is one past the last position get_rope_index gives them
+    lead = (block_len - image_tokens) // 4
+    kinds = torch.tensor([0] * lead + [1] * image_tokens + [0] * (block_len - image_tokens - lead))
+    block_positions = get_rope_index(kinds, kinds, 2, torch.tensor([[1, 2 * side, 2 * side]]))
+    span = int(block_positions.max()) + 1
+    assert span == block_len - image_tokens + side
     gen = torch.Generator().manual_seed(seed)
     need = workers * blocks_per_view * (-(-block_len // P) + 1)
     pages = _Pages(need, P, gen)

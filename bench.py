@@ -19,7 +19,12 @@ bytes of a step (each distinct block counted once) or flops of the visible
 (row, key) pairs, see ``async_llm_amd.workloads``, divided by the wall time per
 step.  ``roofline`` prices the attention launches alone, timed with HIP events on
 the stream they are launched on.  ``cpu_baseline`` times the CPU oracle (torch on
-the host cores) on a bounded sample of the same workload.
+the host cores) on a bounded sample of the same workload, and ``parity`` compares the
+GPU's ``out`` / ``lse`` of that very step with the oracle's outputs for the sample (largest
+absolute and relative errors, within tolerance or not) and the planned integer tables of the
+whole workload with the oracle's planner, bit for bit; a workload that differs ends the
+run with a non-zero exit code.  The region of K timed steps is repeated ``REPEATS`` times;
+``ms_per_step`` is the median region and ``ms_per_step_regions`` the fastest and slowest.
 """
 
 from __future__ import annotations
@@ -35,6 +40,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+REPEATS = 5  # timed regions of K steps each; the line reports the median region
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
@@ -82,9 +88,10 @@ def build_workload(name, device, layers, kernel):
     return workloads.plumbing_decode(device, layers=layers, kernel=kernel)
 
 
-def time_attention_kernel(wl, steps, warmup, layers):
-    """Average duration of the attention launch alone (store excluded), HIP
-    events recorded on the stream the kernels run on."""
+def time_attention_kernel(wl, steps, warmup, layers, repeats=1):
+    """Duration of the attention launch alone (store excluded), HIP events recorded on the
+    stream the kernels run on, over ``repeats`` regions of ``steps`` launches.  Returns the
+    average and the median over all launches and the average of every region."""
     import torch
 
     op, meta = wl.op, wl.meta
@@ -92,15 +99,20 @@ def time_attention_kernel(wl, steps, warmup, layers):
     for i in range(warmup):
         op.attend(wl.q, i % layers, meta)
     torch.cuda.synchronize()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    for i in range(steps):
-        starts[i].record(stream)
-        op.attend(wl.q, i % layers, meta)
-        stops[i].record(stream)
-    torch.cuda.synchronize()
-    times = sorted(s.elapsed_time(e) for s, e in zip(starts, stops))
-    return sum(times) / len(times), times[len(times) // 2]
+    times, region_avg = [], []
+    for _ in range(repeats):
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        for i in range(steps):
+            starts[i].record(stream)
+            op.attend(wl.q, i % layers, meta)
+            stops[i].record(stream)
+        torch.cuda.synchronize()
+        region = [s.elapsed_time(e) for s, e in zip(starts, stops)]
+        region_avg.append(sum(region) / len(region))
+        times += region
+    times.sort()
+    return sum(times) / len(times), times[len(times) // 2], region_avg
 
 
 def cpu_baseline(wl, sample):
@@ -108,7 +120,8 @@ def cpu_baseline(wl, sample):
     blocks, same inputs): rotate+store, per-segment attention, merge.  A mixed
     batch takes its first ``sample`` decode rows and its first prefill chunk.
     Returns (seconds per pass, compulsory bytes of the sample, flops of the
-    sample, cores, description, timed passes)."""
+    sample, cores, description, timed passes, outputs): ``outputs`` lists, per part of
+    the sample, ``(first row, rows, out, lse)`` of the oracle's last pass."""
     import torch
 
     from async_llm_amd.shared_cache import WorkerGroup
@@ -139,7 +152,8 @@ def cpu_baseline(wl, sample):
         def run_decode():
             k_rot = rope.rotate(k.view(n, Hkv, D), pos)
             O.store_kv(k_cpu.view(-1, Hkv * D), v_cpu.view(-1, Hkv * D), slots, k_rot.reshape(n, -1), v)
-            return O.forward_decode(plan, q.view(n, Hq, D), k_cpu, v_cpu, rope)[0]
+            out, lse, _ = O.forward_decode(plan, q.view(n, Hq, D), k_cpu, v_cpu, rope)
+            return 0, n, out, lse
 
         runs.append(run_decode)
         for view in group.cache_structure:  # compulsory bytes of the sample: distinct blocks once
@@ -159,7 +173,8 @@ def cpu_baseline(wl, sample):
         def run_prefill():
             k_rot = rope.rotate(kp.view(rows, Hkv, D), pos_p)
             O.store_kv(k_cpu.view(-1, Hkv * D), v_cpu.view(-1, Hkv * D), out_loc, k_rot.reshape(rows, -1), vp)
-            return O.forward_prefill_batch(plan_p, qp.view(rows, Hq, D), k_cpu, v_cpu, rope)[0]
+            out, lse = O.forward_prefill_batch(plan_p, qp.view(rows, Hq, D), k_cpu, v_cpu, rope)
+            return W, rows, out, lse
 
         runs.append(run_prefill)
         for s in specs:
@@ -170,9 +185,10 @@ def cpu_baseline(wl, sample):
             pairs += s.num_new * before + s.num_new * (s.num_new + 1) // 2
         what.append(f"first {n_p} of {len(wl.specs)} prefill requests ({rows} new tokens)")
 
+    outputs = []
+
     def run():
-        for r in runs:
-            r()
+        outputs[:] = [r() for r in runs]
 
     t0 = time.perf_counter()
     run()
@@ -185,7 +201,92 @@ def cpu_baseline(wl, sample):
         times.append(time.perf_counter() - t0)
     t = sorted(times)[len(times) // 2]
     sample_bytes = b_tok * sum(distinct.values())
-    return t, sample_bytes, 4 * D * Hq * pairs, cores, " + ".join(what), reps
+    return t, sample_bytes, 4 * D * Hq * pairs, cores, " + ".join(what), reps, outputs
+
+
+# out / lse tolerances of the parity contract: 2e-2 abs + 1e-2 rel for 16-bit storage, 1e-5 for fp32
+PARITY_TOL = {"bf16": (2e-2, 1e-2), "f16": (2e-2, 1e-2), "f32": (1e-5, 1e-5)}
+
+
+def index_parity(wl) -> bool:
+    """The product's planned integer tables of the WHOLE workload (sub-row owner, rotation
+    position, pad slot, page / slot table, segment lengths) against the oracle's planner:
+    bit for bit."""
+    import torch
+
+    from tests.util import oracle_decode_plan, oracle_prefill_plan
+
+    meta, P = wl.meta, wl.op.page_size
+    sub_worker, sub_loc, slot, kv, M = [], [], [], [], meta.max_segments
+    checks = []
+    W = 0
+    if wl.mode in ("decode", "mixed"):
+        W = wl.group.num_workers
+        d = oracle_decode_plan(wl.group, wl.pending, wl.new_token_slots.cpu(), P)
+        sub_worker += d.sub_worker
+        loc = torch.tensor(d.sub_loc, dtype=torch.int64)
+        sub_loc.append(loc)
+        slot += [p - w * d.max_segments for p, w in zip(d.pad_slot, d.sub_worker)]
+        kv += d.kv_indices + d.aux_slots
+        checks.append((meta.n_main, meta.n_aux) == (d.n_main, d.n_aux))
+        if meta.main_plan is not None and wl.mode == "decode":
+            checks.append(meta.main_plan["seq_lens"].tolist() == d.seq_lens)
+            checks.append(meta.main_plan["last_page_len"].tolist() == d.last_page_len)
+            checks.append(meta.main_plan["indptr"].tolist() == d.kv_indptr)
+            checks.append(M == d.max_segments)
+    if wl.mode in ("prefill", "mixed"):
+        p = oracle_prefill_plan(wl.specs, P)
+        sub_worker += [r + W for r in p.sub_worker]
+        sub_loc.append(p.sub_loc)
+        slot += [s - r * p.max_segments for s, r in zip(p.pad_slot, p.sub_worker)]
+        kv += p.ctx["kv_indices"] + p.own["kv_indices"]
+        checks.append(meta.n_ctx_rows == p.n_ctx_rows)
+        checks.append(meta.last_indices.cpu().tolist()[-len(p.last_indices):] == [i + W for i in p.last_indices])
+        if wl.mode == "prefill":
+            checks.append(meta.main_plan["seq_lens"].tolist() == p.ctx["seq_lens"])
+            checks.append(meta.aux_plan["seq_lens"].tolist() == p.own["seq_lens"])
+            checks.append(meta.main_plan["paged_kv_last_page_len"].tolist() == p.ctx["last_page_len"])
+            checks.append(meta.aux_plan["paged_kv_last_page_len"].tolist() == p.own["last_page_len"])
+            checks.append(M == p.max_segments)
+    use_3d = any(x.dim() == 2 for x in sub_loc)
+    sub_loc = [x if x.dim() == 2 or not use_3d else x.unsqueeze(0).expand(3, -1) for x in sub_loc]
+    exp_loc = torch.cat(sub_loc, dim=1 if use_3d else 0)
+    exp_worker = torch.tensor(sub_worker, dtype=torch.int64)
+    exp_pad = exp_worker * M + torch.tensor(slot, dtype=torch.int64)
+    checks.append(torch.equal(meta.sub_worker.cpu(), exp_worker))
+    checks.append(torch.equal(meta.sub_loc.cpu(), exp_loc))
+    checks.append(torch.equal(meta.pad_slot.cpu(), exp_pad))
+    checks.append(meta.launch.kv_indices.cpu().tolist() == kv)
+    return all(bool(c) for c in checks)
+
+
+def parity_block(wl, outputs, dtype_name):
+    """Largest errors of the product's ``out`` / ``lse`` (one more step on layer 0, whose pool the
+    oracle read) against the oracle's outputs for the rows of the CPU sample."""
+    import torch
+
+    out, lse = wl.op.forward_with_lse(wl.q, wl.k, wl.v, 0, wl.batch)
+    torch.cuda.synchronize()
+    out, lse = out.cpu().double(), lse.cpu().double()
+    atol, rtol = PARITY_TOL[dtype_name]
+    worst = dict(max_abs_out=0.0, max_rel_out=0.0, max_abs_lse=0.0, max_rel_lse=0.0)
+    within, rows_checked = True, 0
+    for first, rows, exp_out, exp_lse in outputs:
+        for name, got, exp in (("out", out[first:first + rows], exp_out.double()),
+                               ("lse", lse[first:first + rows], exp_lse.double())):
+            err = (got - exp.reshape(got.shape)).abs()
+            ref = exp.reshape(got.shape).abs()
+            worst["max_abs_" + name] = max(worst["max_abs_" + name], err.max().item())
+            # relative error where the reference is large enough for the ratio to mean something
+            big = ref > 10 * atol
+            if big.any():
+                worst["max_rel_" + name] = max(worst["max_rel_" + name], (err[big] / ref[big]).max().item())
+            within = within and bool((err <= atol + rtol * ref).all()) and bool(torch.isfinite(got).all())
+        rows_checked += rows
+    block = {k: float("%.3e" % v) for k, v in worst.items()}
+    block.update(within_tol=within, tolerance={"abs": atol, "rel": rtol}, rows_checked=rows_checked,
+                 indices_bit_exact=index_parity(wl))
+    return block
 
 
 def copy_calibration(dev, steps):
@@ -378,17 +479,22 @@ def measure(wl, steps, warmup, layers, cpu_sample, with_cpu, traffic_ok):
     if warmup is None:
         warmup = max(4, steps // 10)
 
-    # whole step (store + attention + merge), wall clock around K steps
+    # whole step (store + attention + merge), wall clock around K steps; the region of K steps is
+    # timed REPEATS times over (a single short region cannot resolve differences of a percent or two:
+    # clock and box drift are of that size) and the line carries the median region and the spread
     for i in range(warmup):
         wl.forward(i % layers)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        wl.forward(i % layers)
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+    regions = []
+    for _ in range(REPEATS):
+        t0 = time.perf_counter()
+        for i in range(steps):
+            wl.forward(i % layers)
+        torch.cuda.synchronize()
+        regions.append((time.perf_counter() - t0) * 1e3 / steps)
+    ms_per_step = sorted(regions)[len(regions) // 2]
 
-    kern_avg_ms, kern_med_ms = time_attention_kernel(wl, steps, warmup, layers)
+    kern_avg_ms, kern_med_ms, kern_regions = time_attention_kernel(wl, steps, warmup, layers, REPEATS)
     counts = wl.meta.launch.counts
     family = {1: "generic", 2: "mfma"}.get(counts.kernel)
     decode = wl.mode in ("decode", "mixed")  # the mixed batch is priced against HBM, its binding roof
@@ -409,12 +515,15 @@ def measure(wl, steps, warmup, layers, cpu_sample, with_cpu, traffic_ok):
         roof["traffic"] = measured["bytes"]
         roof["traffic_source"] = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, sources " + measured["csrc"]
     roof.update(kernel="attention launch (all work items) + merge", kernel_ms_avg=round(kern_avg_ms, 4),
-                kernel_ms_median=round(kern_med_ms, 4))
+                kernel_ms_median=round(kern_med_ms, 4),
+                kernel_ms_regions=[round(min(kern_regions), 4), round(max(kern_regions), 4)])
     dtype = (str(wl.op.dtype).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32")
              .replace("float16", "f16"))
     line = {
         "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": steps,
-        "warmup": warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "warmup": warmup, "ms_per_step": round(ms_per_step, 4), "repeats": REPEATS,
+        "ms_per_step_regions": [round(min(regions), 4), round(max(regions), 4)],
+        "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dtype, "data": "synthetic",
         "config": {"workload": wl.name, "rows": wl.info.get("rows"), "q_heads": wl.op.num_qo_heads,
                    "kv_heads": wl.op.num_kv_heads, "head_dim": wl.op.head_dim, "page_size": wl.op.page_size,
@@ -426,7 +535,7 @@ def measure(wl, steps, warmup, layers, cpu_sample, with_cpu, traffic_ok):
     }
     if with_cpu:
         sample = cpu_sample or {"decode": 64, "prefill": 1, "mixed": 8}[wl.mode]
-        t_cpu, sample_bytes, sample_flops, cores, what, reps = cpu_baseline(wl, sample)
+        t_cpu, sample_bytes, sample_flops, cores, what, reps, outputs = cpu_baseline(wl, sample)
         if decode:
             cpu_value, cpu_unit = sample_bytes / t_cpu / 1e9, "GB/s"
         else:
@@ -435,6 +544,9 @@ def measure(wl, steps, warmup, layers, cpu_sample, with_cpu, traffic_ok):
                                 "cpu_model": cpu_model(), "kind": "port",
                                 "sample": what + f", {t_cpu:.2f} s per pass, torch CPU oracle, "
                                 + ("median of 3" if reps == 3 else "one pass after one warm-up" if reps == 1 else f"{reps} passes")}
+        # the oracle's outputs of that sample double as the parity check of this very run
+        line["parity"] = parity_block(wl, outputs, dtype)
+        line["parity"]["sample"] = what
     return line
 
 
@@ -492,7 +604,8 @@ def main() -> int:
                 "rows": sub["config"]["rows"], "work_items": sub["config"]["work_items"],
                 "wide_items": sub["config"]["wide_items"], "partials": sub["config"]["partials"],
                 "host_prepare_ms": sub["config"]["host_prepare_ms"], "roofline": sub["roofline"],
-                "cpu_baseline": sub.get("cpu_baseline")}
+                "ms_per_step_regions": sub["ms_per_step_regions"], "repeats": sub["repeats"],
+                "cpu_baseline": sub.get("cpu_baseline"), "parity": sub.get("parity")}
         print(json.dumps(line), flush=True)
         return 0
 
@@ -513,6 +626,10 @@ def main() -> int:
     wl = build_workload(args.workload, dev, args.layers, args.kernel)
     line = measure(wl, args.steps, args.warmup, args.layers, args.cpu_sample, not args.no_cpu_baseline, traffic_ok)
     print(json.dumps(line), flush=True)
+    parity = line.get("parity")
+    if parity and not (parity["within_tol"] and parity["indices_bit_exact"]):
+        print("bench.py: %s differs from the oracle: %s" % (args.workload, json.dumps(parity)), file=sys.stderr)
+        return 3
     return 0
 
 

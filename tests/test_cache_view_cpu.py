@@ -155,3 +155,46 @@ def test_op_refuses_a_pool_whose_layers_are_not_plain_paged_arrays():
         build(torch.zeros(8, 4, 2, 32, dtype=torch.bfloat16)[..., :16])
     with pytest.raises(ValueError, match="contiguous"):
         build(torch.zeros(8, 4, 2, 16, dtype=torch.float16))
+
+
+def test_get_rope_index_known_answers_and_reference_fixtures():
+    """The product's ``get_rope_index`` (reference ``models/qwen3_5_mrope.py:19-64``) against the
+    known answers of the reference's ``tests/core/test_qwen3_5_vision_encoder.py:70-92`` and the
+    HF-generated position fixtures the reference holds (``tests/resources/qwen3_5_0.8B_ref*.npz``,
+    kept here as ``tests/golden/mrope_positions.json``)."""
+    import json
+    import os
+
+    from async_llm_amd.shared_cache.mrope import get_rope_index
+
+    ids = torch.zeros(5, dtype=torch.int64)
+    pos = get_rope_index(ids, torch.zeros(5, dtype=torch.int64), 2)
+    assert torch.equal(pos, torch.arange(5).view(1, -1).expand(3, -1))
+    kinds = torch.tensor([0, 0, 1, 1, 1, 1, 0, 0, 0])
+    pos = get_rope_index(torch.zeros(9, dtype=torch.int64), kinds, 2, torch.tensor([[1, 4, 4]]))
+    assert pos.shape == (3, 9)
+    assert pos[0].tolist() == [0, 1, 2, 2, 2, 2, 4, 5, 6]
+    assert pos[1].tolist() == [0, 1, 2, 2, 3, 3, 4, 5, 6]
+    assert pos[2].tolist() == [0, 1, 2, 3, 2, 3, 4, 5, 6]
+    with pytest.raises(NotImplementedError):
+        get_rope_index(torch.zeros(2, dtype=torch.int64), torch.tensor([0, 7]), 2)
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mrope_positions.json")) as f:
+        cases = json.load(f)
+    assert cases
+    for case in cases:
+        kinds = torch.tensor(case["mm_token_type_ids"])
+        got = get_rope_index(torch.zeros_like(kinds), kinds, case["spatial_merge_size"],
+                             torch.tensor(case["image_grid_thw"]))
+        assert got.tolist() == case["rope_positions"], case["source"]
+
+
+def test_image_block_span_of_the_long_context_workload():
+    """The mRoPE decode workload takes its block span from ``get_rope_index``: a 4096-token image
+    on a 64 x 64 lattice advances the running position by 64 only."""
+    from async_llm_amd.shared_cache.mrope import get_rope_index
+
+    kinds = torch.tensor([0] * 100 + [1] * 4096 + [0] * 50)
+    pos = get_rope_index(kinds, kinds, 2, torch.tensor([[1, 128, 128]]))
+    assert int(pos.max()) + 1 == 100 + 64 + 50
+    assert pos[:, 100].tolist() == [100, 100, 100] and pos[:, 100 + 4095].tolist() == [100, 163, 163]
+    assert pos[:, 100 + 4096].tolist() == [164, 164, 164]

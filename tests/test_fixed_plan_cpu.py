@@ -97,6 +97,43 @@ def test_capacity_holds_chains_packed_in_bundles(heads):
         check_coverage(blob, qo, kvp, lens, flags, sw, n_rows, fixed=True)
 
 
+@pytest.mark.parametrize("heads", [(32, 8, 128), (16, 4, 256)])
+@pytest.mark.parametrize("target", [0, 1, 8, 16])
+def test_capacity_holds_one_row_chunks_over_long_views_beside_a_short_wide_chunk(heads, target):
+    """A short wide chunk next to chunks of one new token over long views: the budget that cuts the
+    narrow tiles' walks must follow THEIR tokens.  Sized from the wide chunk's few tokens it cut
+    every long walk into pieces of the minimum size -- hundreds of items where the capacity derived
+    from the limits (narrow items <= chains + target) has room for a few dozen."""
+    page = 16
+    chains_spec = [(64, [5])] + [(1, [30000] * 4)] * 4
+    qo, kvp, kvi, lens, flags, chain, sw = [0], [0], [], [], [], [], []
+    n_rows, members = 0, 1
+    for r, (new_tokens, context) in enumerate(chains_spec):
+        rows = list(range(n_rows, n_rows + new_tokens))
+        n_rows += new_tokens
+        members = max(members, len(context) + 1)
+        for length in context + [new_tokens]:
+            kvi += list(range(len(kvi), len(kvi) + -(-length // page)))
+            kvp.append(len(kvi)); lens.append(length); chain.append(r); flags.append(0)
+            sw += rows; qo.append(len(sw))
+        flags[-1] = 1
+    tables = (qo, kvp, kvi, lens, flags, chain, sw, n_rows)
+    limits = native.VaPlanLimits(0, 0, len(chains_spec), members, n_rows, n_rows)
+    rc, blob, counts, cap = fixed_plan(tables, limits, heads=heads, page=page, dtype=native.VA_BF16,
+                                       kernel=native.VA_KERNEL_MFMA, target=target)
+    assert rc == 0, native.lib.va_last_error()
+    check_coverage(blob, qo, kvp, lens, flags, sw, n_rows, fixed=True)
+    # the packed plan of the same tables keeps to the same bound: no row with thousands of states
+    arr = [np.ascontiguousarray(a, dtype=np.int32) for a in (qo, kvp, kvi, lens, flags, chain)]
+    swa = np.ascontiguousarray(sw, dtype=np.int64)
+    subs = native.VaSubRequests(len(lens), len(swa), n_rows, arr[0].ctypes.data, arr[1].ctypes.data, arr[2].ctypes.data,
+                                arr[3].ctypes.data, arr[4].ctypes.data, arr[5].ctypes.data, swa.ctypes.data)
+    packed = native.VaPlanCounts()
+    assert native.lib.va_plan_count(subs, native.VaShape(heads[0], heads[1], heads[2], page, native.VA_BF16),
+                                    native.VaPlanParams(native.VA_KERNEL_MFMA, 0, 0, target, 0), packed) == 0
+    assert packed.n_items - packed.n_wide_items <= cap.max_items
+
+
 def test_padding_per_die_never_exceeds_a_capacity_the_real_items_fit():
     """One heavy unit and many light ones: dealing by load alone gives one die few
     entries and the others many, and padding every die to the longest list would
@@ -203,7 +240,7 @@ def test_decode_buffers_keep_the_reference_geometry():
     h, items, links, *_ = decode_plan(buffers._blob_host.numpy())
     packed = decode_plan(plain.launch.blob.numpy())
     assert sorted(int(i[4]) for i in items if i[2]) == sorted(int(i[4]) for i in packed[1] if i[2])
-    assert buffers.workspace_requirements() == [buffers.counts.workspace_bytes]
+    assert buffers.workspace_requirements() == [(buffers, buffers.counts.workspace_bytes, 0)]
 
 
 def test_decode_buffers_capacity_errors():
@@ -291,12 +328,83 @@ def test_prepare_workspace_takes_the_largest_profile():
     att = make_attention(4)
     small = SharedDecodeAttentionBuffers(att, workers=2, depth=2, max_pages=8)
     large = SharedPrefillAttentionBuffers(att, workers=2, depth=2, rows=64, max_pages=64)
-    need = max(small.workspace_requirements() + large.workspace_requirements())
+    need = max(entry[1] for entry in small.workspace_requirements() + large.workspace_requirements())
+    assert need == max(large.counts.workspace_bytes, small.counts.workspace_bytes) > 0
     att._workspace = None
     att.prepare_workspace([small, large])
     assert att._workspace.numel() == need
+    # both profiles launch out of the one arena
+    assert small.meta.launch.workspace is att._workspace and large.meta.launch.workspace is att._workspace
     with pytest.raises(RuntimeError, match="prepared once"):
         att.prepare_workspace([small])
     other = make_attention(4)
     with pytest.raises(ValueError, match="belong to this instance"):
         other.prepare_workspace([small])
+
+
+def bare_attention(monkeypatch):
+    """An op with nothing but its workspace state, as the reference's workspace tests build one
+    (``tests/core/test_attention_workspace.py:14-20``)."""
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: False)
+    att = SharedCacheAttention.__new__(SharedCacheAttention)
+    att.device = CPU
+    att._workspace = torch.empty(8, dtype=torch.uint8)
+    att._workspace_prepared = False
+    return att
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_catalogue_shares_the_largest_arena_but_not_the_table_storage(monkeypatch, reverse):
+    # known answers of the reference's tests/core/test_attention_workspace.py:23-41
+    att = bare_attention(monkeypatch)
+    consumers = [SimpleNamespace() for _ in range(4)]
+    for c in consumers:
+        def reset(arena, ints, c=c):
+            c.arena, c.ints = arena, ints
+        c.reset_workspace_buffer = reset
+    decode = SimpleNamespace(attention=att, workspace_requirements=lambda: [(consumers[0], 32, 24), (consumers[1], 16, 0)])
+    prefill = SimpleNamespace(attention=att, workspace_requirements=lambda: [(consumers[2], 64, 48), (consumers[3], 8, 16)])
+    att.prepare_workspace([prefill, decode] if reverse else [decode, prefill])
+    assert att._workspace.numel() == 64
+    assert all(c.arena is att._workspace for c in consumers)
+    assert [c.ints.numel() for c in consumers] == [24, 16, 48, 16]
+    assert len({c.ints.data_ptr() for c in consumers}) == 4
+    with pytest.raises(RuntimeError, match="once before capture"):
+        att.prepare_workspace([decode])
+
+
+def test_failed_allocation_or_capture_rebinds_nothing(monkeypatch):
+    # the scenario of the reference's tests/core/test_attention_workspace.py:44-68: the third
+    # allocation (arena, first table, SECOND table) fails
+    att = bare_attention(monkeypatch)
+    original = att._workspace
+    calls = []
+    consumer = SimpleNamespace(reset_workspace_buffer=lambda *args: calls.append(args))
+    profile = SimpleNamespace(attention=att, workspace_requirements=lambda: [(consumer, 64, 24), (consumer, 32, 48)])
+    real_empty, count = torch.empty, 0
+
+    def allocate(*args, **kwargs):
+        nonlocal count
+        count += 1
+        if count == 3:
+            raise torch.OutOfMemoryError("test allocation")
+        return real_empty(*args, **kwargs)
+
+    with monkeypatch.context() as patch:
+        patch.setattr(torch, "empty", allocate)
+        with pytest.raises(torch.OutOfMemoryError):
+            att.prepare_workspace([profile])
+    assert not calls and att._workspace is original and not att._workspace_prepared
+    att.device = torch.device("cuda")  # capture is only ever asked about on a GPU op
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
+    with pytest.raises(RuntimeError, match="before capture"):
+        att.prepare_workspace([profile])
+    assert not calls and not att._workspace_prepared
+
+
+def test_empty_catalogue_and_foreign_owner(monkeypatch):
+    att = bare_attention(monkeypatch)
+    att.prepare_workspace([])
+    assert not att._workspace_prepared
+    with pytest.raises(ValueError, match="belong"):
+        att.prepare_workspace([SimpleNamespace(attention=object())])

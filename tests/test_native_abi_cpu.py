@@ -15,7 +15,8 @@ from async_llm_amd import native
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 H = dict(MAGIC=0, KERNEL=1, Q_TILE=2, KV_CHUNK=3, N_ITEMS=4, N_LINKS=5, N_QREFS=6, N_PARTIALS=7, N_ROW_PARTS=8,
          N_ROWS=9, OFF_ITEMS=10, OFF_LINKS=11, OFF_QREFS=12, OFF_ROW_INDPTR=13, OFF_ROW_IDS=14, OFF_ROW_FLAGS=15,
-         N_EMPTY=16, N_SUBROWS=17, N_WIDE=18, WIDE_TILE=19, OFF_QREF_ROWS=20, N_WIDE_SLOTS=21, OFF_WIDE_SLOTS=22)
+         N_EMPTY=16, N_SUBROWS=17, N_WIDE=18, WIDE_TILE=19, OFF_QREF_ROWS=20, N_WIDE_SLOTS=21, OFF_WIDE_SLOTS=22,
+         MERGE_WAVES=23)
 NO_CAUSAL = 0x3FFFFFFF
 
 
@@ -81,6 +82,10 @@ def check_coverage(blob, qo, kvp, lens, flags, sub_worker, n_rows, fixed=False):
     # the wide launch runs one workgroup per slot: the slots partition the real wide items, in order
     slots = blob[h[H["OFF_WIDE_SLOTS"]]: h[H["OFF_WIDE_SLOTS"]] + h[H["N_WIDE_SLOTS"]] + 1]
     assert h[H["N_WIDE_SLOTS"]] % 8 == 0 and slots[0] == 0 and all(a <= b for a, b in zip(slots, slots[1:]))
+    # waves per merge workgroup: by the states per row, one wave when the rows are many
+    n_rows_h, per_row = max(1, int(h[H["N_ROWS"]])), int(h[H["N_ROW_PARTS"]]) // max(1, int(h[H["N_ROWS"]]))
+    assert h[H["MERGE_WAVES"]] in (1, 4, 8, 16)
+    assert (h[H["MERGE_WAVES"]] == 16) == (per_row >= 48) or h[H["MERGE_WAVES"]] == 1
     assert slots[-1] <= h[H["N_WIDE"]] and all(it[2] == 0 for it in items[slots[-1]: h[H["N_WIDE"]]])
     for it in items:
         lb, nl, nq, part_base = it[0], it[1], it[2], it[3]

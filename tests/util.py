@@ -85,10 +85,26 @@ def make_op_and_pool(device, dtype, heads, page, num_pages, theta, rotary_dim=No
     return op, (k_cpu, v_cpu), (k_dev, v_dev), g
 
 
+def fused_rows(dev, *parts):
+    """The rows of ``parts`` (CPU tensors ``[N, width_i]``) as column slices of ONE device tensor
+    ``[N, sum(width_i) + gap]``, the way an attention layer hands q, k and v to the op: views into
+    its fused qkv projection, row stride = the projection's width (reference
+    ``layers/attention.py:47-64``)."""
+    gap = 64  # unrelated columns, poisoned: a kernel that ignored the row stride would read them
+    fused = torch.cat(list(parts) + [torch.full((parts[0].shape[0], gap), float("nan"), dtype=parts[0].dtype)], dim=1).to(dev)
+    views, at = [], 0
+    for part in parts:
+        views.append(fused[:, at:at + part.shape[1]])
+        at += part.shape[1]
+    assert all(not v.is_contiguous() or v.shape[0] <= 1 for v in views)
+    return views
+
+
 def run_decode_parity(op, cpu_pool, dev_pool, group, page_alloc, theta, gen, scale=None, check_pool_exact=True,
-                      lse_base2=False):
+                      lse_base2=False, fused_qkv=False):
     """One decode step through the product op and through the oracle; returns
-    the product and oracle outputs after asserting parity."""
+    the product and oracle outputs after asserting parity.  ``fused_qkv``: q, k and v reach
+    the op as row-strided slices of one tensor."""
     from types import SimpleNamespace
 
     from async_llm_amd.shared_cache.session_planning import plan_decode_writes
@@ -106,7 +122,8 @@ def run_decode_parity(op, cpu_pool, dev_pool, group, page_alloc, theta, gen, sca
     v = (torch.randn(W, Hkv * D, generator=gen) * scale).to(op.dtype)
     positions = torch.tensor(write_pos, dtype=torch.int64)
     batch = SimpleNamespace(attn_metadata=meta, positions=positions.to(dev), out_loc=slots, mrope_positions=None)
-    out, lse = op.forward_with_lse(q.to(dev), k.to(dev), v.to(dev), 0, batch, lse_base2=lse_base2)
+    q_dev, k_dev, v_dev = fused_rows(dev, q, k, v) if fused_qkv else (q.to(dev), k.to(dev), v.to(dev))
+    out, lse = op.forward_with_lse(q_dev, k_dev, v_dev, 0, batch, lse_base2=lse_base2)
     torch.cuda.synchronize()
 
     rope = oracle_rope(op, theta)
@@ -166,9 +183,10 @@ def oracle_prefill(op, cpu_pool, specs, theta, positions, mrope_positions, out_l
     return O.forward_prefill_batch(oracle_prefill_plan(specs, P), q.view(N, Hq, D), k_cpu, v_cpu, rope)
 
 
-def run_prefill_parity(op, cpu_pool, dev_pool, specs, theta, gen, scale=None, mutate=None):
+def run_prefill_parity(op, cpu_pool, dev_pool, specs, theta, gen, scale=None, mutate=None, fused_qkv=False):
     """One batched prefill through the product op and through the oracle.  ``mutate(q, k, v)`` may
-    edit the random input rows (CPU tensors) in place before either side sees them."""
+    edit the random input rows (CPU tensors) in place before either side sees them; ``fused_qkv``:
+    q, k and v reach the op as row-strided slices of one tensor."""
     from types import SimpleNamespace
 
     dev = op.device
@@ -182,7 +200,8 @@ def run_prefill_parity(op, cpu_pool, dev_pool, specs, theta, gen, scale=None, mu
         mutate(q, k, v)
     batch = SimpleNamespace(attn_metadata=meta, positions=positions.to(dev), out_loc=out_loc.to(dev),
                             mrope_positions=None if mrope_positions is None else mrope_positions.to(dev))
-    out, lse = op.forward_with_lse(q.to(dev), k.to(dev), v.to(dev), 0, batch)
+    q_dev, k_dev, v_dev = fused_rows(dev, q, k, v) if fused_qkv else (q.to(dev), k.to(dev), v.to(dev))
+    out, lse = op.forward_with_lse(q_dev, k_dev, v_dev, 0, batch)
     torch.cuda.synchronize()
 
     exp_out, exp_lse = oracle_prefill(op, cpu_pool, specs, theta, positions, mrope_positions, out_loc, q, k, v)
