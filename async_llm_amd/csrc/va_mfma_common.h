@@ -214,8 +214,13 @@ constexpr int kAccumulatorWaitStates = kMfma32Passes + 3 + 4;
 static_assert(kAccumulatorWaitStates <= 16, "one s_nop holds at most 16 wait states");
 template <int kCount>
 __device__ __forceinline__ void accumulator_fence(va_f32x16* o) {
-  static_assert(kCount == 2 || kCount == 4 || kCount == 8, "accumulators per wave");
-  if constexpr (kCount == 8) {
+  static_assert(kCount == 2 || kCount == 4 || kCount == 8 || kCount == 16, "accumulators per wave");
+  if constexpr (kCount == 16) {
+    asm volatile("s_nop %16"
+                 : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(o[4]), "+a"(o[5]), "+a"(o[6]), "+a"(o[7]),
+                   "+a"(o[8]), "+a"(o[9]), "+a"(o[10]), "+a"(o[11]), "+a"(o[12]), "+a"(o[13]), "+a"(o[14]), "+a"(o[15])
+                 : "n"(kAccumulatorWaitStates - 1));
+  } else if constexpr (kCount == 8) {
     asm volatile("s_nop %8"
                  : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(o[4]), "+a"(o[5]), "+a"(o[6]), "+a"(o[7])
                  : "n"(kAccumulatorWaitStates - 1));

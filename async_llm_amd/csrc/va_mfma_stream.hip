@@ -412,6 +412,15 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
 template <typename E, int kD>
 static int launch_stream_one(const AttnArgs& a, int n_items, hipStream_t stream) {
   const dim3 grid((unsigned)n_items * (unsigned)a.num_kv_heads), block(kStreamThreads);
+  if constexpr (StreamShape<kD>::kLdsBytes > 64 * 1024) {  // (deeper rings than the default need the limit raised)
+    static bool configured = false;  // raising the limit is idempotent; a race only repeats the call
+    if (!configured) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_stream_kernel<E, kD>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, StreamShape<kD>::kLdsBytes);
+      if (e != hipSuccess) return va_fail(VA_ERR_HIP, "raising the LDS limit: %s", hipGetErrorString(e));
+      configured = true;
+    }
+  }
   hipLaunchKernelGGL((attn_stream_kernel<E, kD>), grid, block, StreamShape<kD>::kLdsBytes, stream, a);
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? VA_OK : va_fail(VA_ERR_HIP, "streaming attention launch: %s", hipGetErrorString(e));
