@@ -267,6 +267,19 @@ __device__ __forceinline__ void load_to_lds(const void* src, uint32_t lds_base) 
       : "v"(src), "s"(lds_base)
       : "memory");
 }
+// The same load marked non-temporal: rows that one workgroup reads once (a block no other query
+// tile shares) are streamed through the caches as lines to evict first, so that they do not push
+// out the rows that several tiles read (a block shared by many views, held in the die's L2).
+__device__ __forceinline__ void load_to_lds_once(const void* src, uint32_t lds_base) {
+  uint32_t saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, off nt\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(src), "s"(lds_base)
+      : "memory");
+}
 // The same with a wave-uniform base address and a 32-bit per-lane byte offset (no vector ALU work
 // to form 64-bit addresses).
 __device__ __forceinline__ void load_to_lds(const void* base, uint32_t lane_offset, uint32_t lds_base) {

@@ -177,6 +177,8 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     const int tok_end = link[VA_L_TOK_END];
     const int causal_base = link[VA_L_CAUSAL_BASE];
     const bool slots = lflags & VA_LINK_SLOTS;
+    // no other query tile reads these rows: they are requested as lines to evict first
+    const bool read_once = lflags & VA_LINK_ONCE;
     // a 16-token tile lies inside one page: one wave-uniform page read per tile
     const bool uniform_pages = !slots && pow2_pages && P >= 16 && (tok_begin % 16 == 0);
 
@@ -193,8 +195,9 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     auto page_of = [&](int i) __attribute__((always_inline)) {
       return ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + ((tok_begin + i * kStreamTok) >> p_shift)];
     };
-    auto issue = [&](int i, auto uniform_tag, int page) __attribute__((always_inline)) {
+    auto issue = [&](int i, auto uniform_tag, auto once_tag, int page) __attribute__((always_inline)) {
       constexpr bool kUniform = decltype(uniform_tag)::value;
+      constexpr bool kOnce = decltype(once_tag)::value;
       const int t0 = tok_begin + i * kStreamTok;
       va_u32x4* buf = ring + (i % kBuffers) * 2 * kTileUnits;
       long long base_byte = 0;  // wave-uniform: pool byte offset of the tile's first token
@@ -216,22 +219,39 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
                 ld_byte[u];
         }
         const va_u32x4* dst = buf + (is_v ? kTileUnits : 0) + first_row * kChunks;  // + lane, implied by the load
-        load_to_lds(src, __builtin_amdgcn_readfirstlane(lds_address(dst)));
+        if constexpr (kOnce) {
+          load_to_lds_once(src, __builtin_amdgcn_readfirstlane(lds_address(dst)));
+        } else {
+          load_to_lds(src, __builtin_amdgcn_readfirstlane(lds_address(dst)));
+        }
       }
     };
 
     // ---- set-up: first tiles on their way, then the query tile ----
     __syncthreads();  // every wave is done with the previous link's buffers
-    auto first_tiles = [&](auto uniform_tag) __attribute__((always_inline)) {
+    auto first_tiles = [&](auto uniform_tag, auto once_tag) __attribute__((always_inline)) {
 #pragma unroll
       for (int i = 0; i < kBuffers - 1; ++i)
-        if (i < n_tiles) issue(i, uniform_tag, decltype(uniform_tag)::value ? page_of(i) : 0);
+        if (i < n_tiles) issue(i, uniform_tag, once_tag, decltype(uniform_tag)::value ? page_of(i) : 0);
     };
-    if (uniform_pages) {
-      first_tiles(std::true_type{});
-    } else {
-      first_tiles(std::false_type{});
-    }
+    // (one instance of the requests and of the tile loop per page-table kind and per cache policy,
+    // so that none carries the others' branches)
+    auto per_kind = [&](auto&& body) __attribute__((always_inline)) {
+      if (uniform_pages) {
+        if (read_once) {
+          body(std::true_type{}, std::true_type{});
+        } else {
+          body(std::true_type{}, std::false_type{});
+        }
+      } else {
+        if (read_once) {
+          body(std::false_type{}, std::true_type{});
+        } else {
+          body(std::false_type{}, std::false_type{});
+        }
+      }
+    };
+    per_kind(first_tiles);
 
     // rotate the query tile into the last buffer (not yet in use), swizzled like a K tile
     va_u32x4* q_stage = ring + (kBuffers - 1) * 2 * kTileUnits;
@@ -267,9 +287,9 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
     for (int s = 0; s < kSteps; ++s) qf[s] = q_stage[j * kChunks + ((4 * s + kg) ^ swz<kD>(j))];
     ring_barrier<kAnyInFlight>();  // the staging buffer may be refilled now
 
-    // ---- the tile loop, once per page-table kind so neither carries the other's branches ----
-    auto stream = [&](auto uniform_tag) __attribute__((always_inline)) {
-    if (kBuffers - 1 < n_tiles) issue(kBuffers - 1, uniform_tag, decltype(uniform_tag)::value ? page_of(kBuffers - 1) : 0);
+    // ---- the tile loop ----
+    auto stream = [&](auto uniform_tag, auto once_tag) __attribute__((always_inline)) {
+    if (kBuffers - 1 < n_tiles) issue(kBuffers - 1, uniform_tag, once_tag, decltype(uniform_tag)::value ? page_of(kBuffers - 1) : 0);
     for (int i = 0; i < n_tiles; ++i) {
       // This wave's loads of tile i have landed once at most the loads of the tiles requested
       // after it are outstanding; the barrier then covers the other waves' loads.
@@ -353,15 +373,11 @@ __global__ __launch_bounds__(kStreamThreads, StreamShape<kD>::kMinBlocks) void a
       // refill this tile's buffer once every wave has consumed it
       if (refill) {
         ring_barrier<kAnyInFlight>();
-        issue(i + kBuffers, uniform_tag, next_page);
+        issue(i + kBuffers, uniform_tag, once_tag, next_page);
       }
     }
     };
-    if (uniform_pages) {
-      stream(std::true_type{});
-    } else {
-      stream(std::false_type{});
-    }
+    per_kind(stream);
   }
 
   // row sums live spread over the four contraction groups

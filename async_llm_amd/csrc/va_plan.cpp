@@ -280,8 +280,12 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   for (auto& gr : groups) {
     const int32_t rep = gr.rep;
     const int32_t len = s->seq_lens[rep];
-    const int32_t lflags = VA_LINK_INDIRECT | ((s->flags[rep] & VA_SUB_SLOTS) ? VA_LINK_SLOTS : 0);
     cut_tiles((int64_t)gr.subrows.size(), tiles, wide_groups);
+    // A run that a single query tile reads is fetched once per kv head and never again: its rows are
+    // requested as lines to evict first, so that they stream through the die's L2 without pushing
+    // out the rows that several tiles read side by side (a block shared by many views).
+    const int32_t lflags = VA_LINK_INDIRECT | ((s->flags[rep] & VA_SUB_SLOTS) ? VA_LINK_SLOTS : 0) |
+                           (tiles.size() == 1 ? VA_LINK_ONCE : 0);
     std::vector<int32_t> tile_qref;
     for (auto& tl : tiles) {
       tile_qref.push_back((int32_t)out.qrefs.size());

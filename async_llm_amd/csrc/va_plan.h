@@ -65,6 +65,8 @@ enum {
 
 #define VA_LINK_INDIRECT 1  // sub-row of tile row i is qrefs[qref + i], else qref + i
 #define VA_LINK_SLOTS 2     // kv_indices entries are token slots (page size 1)
+#define VA_LINK_ONCE 4      // no other query tile of the launch reads this token range (per kv head the rows are
+                            // fetched exactly once): the streaming kernel requests them non-temporally
 
 #define VA_NO_CAUSAL 0x3fffffff
 
