@@ -36,11 +36,15 @@ struct alignas(kVec * sizeof(S) == 16 ? 16 : alignof(S)) Piece {
   S v[kVec];
 };
 
+// 16-byte pieces travel as non-temporal loads and stores: every row is read once and written once,
+// nothing of it is worth a place in the caches (two 16 384-token blocks over four layers: 259 -> 247 us).
+typedef uint32_t va_copy_u32x4 __attribute__((ext_vector_type(4)));
+
 template <typename S, int kVec>
 __device__ __forceinline__ Piece<S, kVec> load_piece(const S* p) {
   Piece<S, kVec> out;
   if constexpr (kVec * sizeof(S) == 16) {
-    *reinterpret_cast<uint4*>(out.v) = *reinterpret_cast<const uint4*>(p);
+    *reinterpret_cast<va_copy_u32x4*>(out.v) = __builtin_nontemporal_load(reinterpret_cast<const va_copy_u32x4*>(p));
   } else {
 #pragma unroll
     for (int i = 0; i < kVec; ++i) out.v[i] = p[i];
@@ -51,7 +55,7 @@ __device__ __forceinline__ Piece<S, kVec> load_piece(const S* p) {
 template <typename S, int kVec>
 __device__ __forceinline__ void store_piece(S* p, const Piece<S, kVec>& x) {
   if constexpr (kVec * sizeof(S) == 16) {
-    *reinterpret_cast<uint4*>(p) = *reinterpret_cast<const uint4*>(x.v);
+    __builtin_nontemporal_store(*reinterpret_cast<const va_copy_u32x4*>(x.v), reinterpret_cast<va_copy_u32x4*>(p));
   } else {
 #pragma unroll
     for (int i = 0; i < kVec; ++i) p[i] = x.v[i];

@@ -270,6 +270,8 @@ __device__ __forceinline__ void load_to_lds(const void* src, uint32_t lds_base) 
 // The same load marked non-temporal: rows that one workgroup reads once (a block no other query
 // tile shares) are streamed through the caches as lines to evict first, so that they do not push
 // out the rows that several tiles read (a block shared by many views, held in the die's L2).
+// Measured on one MI355X: a pure stream (eight views of 131 072 tokens, nothing shared) 5.74 -> 6.29 TB/s;
+// it is the nt bit that does it, the sc0 / sc1 bits beside it change nothing.
 __device__ __forceinline__ void load_to_lds_once(const void* src, uint32_t lds_base) {
   uint32_t saved;
   asm volatile(
