@@ -236,7 +236,13 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   int32_t kv_chunk = params && params->kv_chunk > 0 ? round_up(params->kv_chunk, gran) : 0;
   if (kv_chunk == 0) {
     const int64_t per_item = (total_tokens + target - 1) / target;
-    kv_chunk = round_up(std::max<int64_t>(per_item, 4 * gran), gran);
+    // No chunk under four granules as a rule (an item's set-up is worth a few hundred tokens) -- unless the
+    // launch holds so few tokens that such chunks would leave most of the machine idle: then the time of
+    // the launch is the walk of ONE item, a chain of dependent trips to memory, and shorter walks side by
+    // side (down to one granule) are what shortens it.
+    const int64_t spread = (total_tokens + (256 / shape->num_kv_heads) - 1) / std::max(1, 256 / shape->num_kv_heads);
+    const int64_t least = std::min<int64_t>(4 * gran, std::max<int64_t>(gran, round_up(spread, gran)));
+    kv_chunk = round_up(std::max<int64_t>(per_item, least), gran);
   }
 
   out.kernel = kernel;

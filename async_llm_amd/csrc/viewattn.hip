@@ -246,6 +246,7 @@ int launch_rope_store(const void* x, const void* v, void* y, void* v_out, long l
 constexpr int kHB = 4;          // q heads per pass
 constexpr int kGenThreads = 256;
 constexpr int kGenWaves = kGenThreads / kWave;
+constexpr int kGenAhead = 4;     // steps of the token walk whose loads are in flight together
 
 template <typename E, int kD>
 __global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
@@ -322,42 +323,59 @@ __global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
         const int t_end = min(link[VA_L_TOK_END], link[VA_L_CAUSAL_BASE] + iq + 1);
         const int kv_begin = link[VA_L_KV_BEGIN];
         const bool slots = lflags & VA_LINK_SLOTS;
-        for (int t0 = link[VA_L_TOK_BEGIN] + wave * kTPW; t0 < t_end; t0 += kGenWaves * kTPW) {
-          const int t = t0 + lg;
-          const bool live = t < t_end;
-          float sc[kHB];
-          uint4 kraw = make_uint4(0, 0, 0, 0), vraw = make_uint4(0, 0, 0, 0);
-          if (live) {
-            const long long slot = kv_slot(a.kv_indices, kv_begin, t, a.page_size, slots);
-            const long long off = slot * a.pool_row_stride + (long long)hk * kD + li * kVec;
-            kraw = *(const uint4*)(kp + off);
-            vraw = *(const uint4*)(vp + off);
-          }
-          const S* ke = (const S*)&kraw;
-          const S* ve = (const S*)&vraw;
-          float kf[kVec], vf[kVec];
+        // kGenAhead steps of the walk at a time: their page lookups first, then their K and V rows, all
+        // in flight together -- a step by itself is a chain of two dependent trips to memory, and at
+        // decode sizes (a few hundred tokens per workgroup) the kernel is nothing but that chain
+        for (int t0 = link[VA_L_TOK_BEGIN] + wave * kTPW; t0 < t_end; t0 += kGenAhead * kGenWaves * kTPW) {
+          bool live[kGenAhead];
+          long long off[kGenAhead];
+          uint4 kraw[kGenAhead], vraw[kGenAhead];
 #pragma unroll
-          for (int e = 0; e < kVec; ++e) {
-            kf[e] = E::load(ke[e]);
-            vf[e] = E::load(ve[e]);
+          for (int u = 0; u < kGenAhead; ++u) {
+            const int t = t0 + u * kGenWaves * kTPW + lg;
+            live[u] = t < t_end;
+            const long long slot = kv_slot(a.kv_indices, kv_begin, live[u] ? t : t_end - 1, a.page_size, slots);
+            off[u] = slot * a.pool_row_stride + (long long)hk * kD + li * kVec;
           }
 #pragma unroll
-          for (int g = 0; g < kHB; ++g) {
-            float d = 0.f;
-#pragma unroll
-            for (int e = 0; e < kVec; ++e) d = fmaf(qr[g][e], kf[e], d);
-            d = group_sum<kLPT>(d);
-            sc[g] = live ? d * a.scale_log2 : -INFINITY;
+          for (int u = 0; u < kGenAhead; ++u) {
+            kraw[u] = make_uint4(0, 0, 0, 0);
+            vraw[u] = make_uint4(0, 0, 0, 0);
+            if (live[u]) {
+              kraw[u] = *(const uint4*)(kp + off[u]);
+              vraw[u] = *(const uint4*)(vp + off[u]);
+            }
           }
 #pragma unroll
-          for (int g = 0; g < kHB; ++g) {
-            const float m_new = fmaxf(m[g], sc[g]);
-            const float alpha = exp2f(m[g] - m_new);
-            const float pr = exp2f(sc[g] - m_new);
-            m[g] = m_new;
-            l[g] = l[g] * alpha + pr;
+          for (int u = 0; u < kGenAhead; ++u) {
+            if (t0 + u * kGenWaves * kTPW >= t_end) break;  // (wave-uniform: the step lies past the range)
+            float sc[kHB];
+            const S* ke = (const S*)&kraw[u];
+            const S* ve = (const S*)&vraw[u];
+            float kf[kVec], vf[kVec];
 #pragma unroll
-            for (int e = 0; e < kVec; ++e) acc[g][e] = fmaf(pr, vf[e], acc[g][e] * alpha);
+            for (int e = 0; e < kVec; ++e) {
+              kf[e] = E::load(ke[e]);
+              vf[e] = E::load(ve[e]);
+            }
+#pragma unroll
+            for (int g = 0; g < kHB; ++g) {
+              float d = 0.f;
+#pragma unroll
+              for (int e = 0; e < kVec; ++e) d = fmaf(qr[g][e], kf[e], d);
+              d = group_sum<kLPT>(d);
+              sc[g] = live[u] ? d * a.scale_log2 : -INFINITY;
+            }
+#pragma unroll
+            for (int g = 0; g < kHB; ++g) {
+              const float m_new = fmaxf(m[g], sc[g]);
+              const float alpha = exp2f(m[g] - m_new);
+              const float pr = exp2f(sc[g] - m_new);
+              m[g] = m_new;
+              l[g] = l[g] * alpha + pr;
+#pragma unroll
+              for (int e = 0; e < kVec; ++e) acc[g][e] = fmaf(pr, vf[e], acc[g][e] * alpha);
+            }
           }
         }
       }

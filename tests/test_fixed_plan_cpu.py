@@ -144,7 +144,7 @@ def test_padding_per_die_never_exceeds_a_capacity_the_real_items_fit():
     def add(n_tokens, first_page, w):
         kvi.extend(range(first_page, first_page + -(-n_tokens // page)))
         kvp.append(len(kvi)); lens.append(n_tokens); flags.append(0); chain.append(-1); sw.append(w); qo.append(len(sw))
-    add(192, 0, 0)  # below four granules: a run this short is not cut
+    add(64, 0, 0)  # one granule: a run this short is never cut
     for w in range(1, 40):
         add(16, 100 + w, w)
     tables = (qo, kvp, kvi, lens, flags, chain, sw, 40)
