@@ -180,6 +180,11 @@ VA_API int va_plan_count(const VaSubRequests* subs, const VaShape* shape, const 
  * row_flags[n_rows] | wide_slots[n_wide_slots+1].  (An item carries a copy of its first link, and qref_rows
  * the output row of every qrefs entry: both shorten the chain of dependent loads
  * at the start of a workgroup.)
+ * A link whose token range no other query tile of the launch reads carries the
+ * flag "read once" (its rows are then requested as non-temporal loads, which
+ * stream through the die's L2 as lines to evict first); the header also holds
+ * the number of waves per workgroup of the merge launch, chosen from the
+ * partial states per row (from the capacity, for a fixed plan).
  * Items are in launch order, laid out for the 8 dies of an MI355X (workgroup b
  * of a launch runs on die b % 8): wide items first, then narrow ones, each
  * class padded with empty items (n_q = 0) to a multiple of 8; n_items and

@@ -281,6 +281,43 @@ def test_tiles_of_one_chunk_run_on_one_die():
     check_coverage(blob, qo, kvp, lens, flags, sw, n_req)
 
 
+def test_runs_that_one_tile_reads_are_flagged_read_once():
+    """Ten requests read one 4096-token block and own a private block each (bf16, 16 q / 4 kv heads: 4 requests
+    fill a 16-row tile).  The shared block is walked by three query tiles, which should find it in the die's
+    L2, so its links stay plain; a private block is read by exactly one tile and streams through the caches
+    once: its links carry the read-once flag (the streaming kernel then requests the rows non-temporally),
+    whether the run is cut into chunks or not."""
+    page, shared_len = 16, 4096
+    shared_pages = list(range(shared_len // page))
+    kvi, kvp, lens, sw = [], [0], [], []
+    next_page = len(shared_pages)
+    private_len = [700, 64, 3000, 1, 16, 900, 2048, 333, 5000, 50]
+    for w, n in enumerate(private_len):
+        kvi += shared_pages; kvp.append(len(kvi)); lens.append(shared_len); sw.append(w)
+        pages = -(-n // page)
+        kvi += list(range(next_page, next_page + pages)); next_page += pages
+        kvp.append(len(kvi)); lens.append(n); sw.append(w)
+    n_sub = len(lens)
+    rc, blob, counts = build_plan(list(range(n_sub + 1)), kvp, kvi, lens, [0] * n_sub, [-1] * n_sub, sw, len(private_len),
+                                  heads=(16, 4, 256), page=page, dtype=native.VA_BF16, kernel=native.VA_KERNEL_MFMA)
+    assert rc == 0
+    check_coverage(blob, list(range(n_sub + 1)), kvp, lens, [0] * n_sub, sw, len(private_len))
+    h, items, links, *_ = decode_plan(blob)
+    ONCE = 4
+    seen = {True: 0, False: 0}
+    for it in items:
+        if not it[2]:
+            continue
+        for l in links[it[0]: it[0] + it[1]]:
+            is_shared = int(l[0]) in [kvp[2 * w] for w in range(len(private_len))] and int(l[2]) - int(l[1]) > 0 and \
+                kvi[int(l[0])] == 0
+            assert bool(int(l[5]) & ONCE) == (not is_shared), (list(l), is_shared)
+            seen[is_shared] += 1
+            # the copy of the first link that travels in the item carries the same flags
+            assert int(it[8 + 5]) == int(links[it[0]][5])
+    assert seen[True] >= 3 and seen[False] >= len(private_len)
+
+
 def test_plan_rejects_inconsistent_tables():
     ok = dict(qo=[0, 1], kvp=[0, 2], kvi=[3, 4], lens=[8], flags=[0], chain=[-1], sub_worker=[0], n_rows=1)
 
