@@ -145,8 +145,13 @@ class SharedCacheAttention:
         mrope_section: tuple | None = None,
         rope_base: float | None = None,
         kernel: str | None = None,
+        fused_store: bool = True,
     ) -> None:
         self.kv_cache = kv_cache
+        # False: new rows reach the pool through ``kv_cache.store_kv`` as in the reference
+        # (``attention.py:645-649``: rotate, then store), one launch more per step -- for a pool whose
+        # ``store_kv`` does more than copy rows (hooks, a storage format of its own behind it)
+        self.fused_store = fused_store
         self.num_qo_heads = num_qo_heads
         self.num_kv_heads = num_kv_heads
         self.head_dim = head_dim
@@ -182,7 +187,8 @@ class SharedCacheAttention:
         self._workspace_prepared = False
         self._plan_scratch = np.empty(1 << 16, dtype=np.int32)  # host scratch of the planner, grown on demand
         self._checked_layers = set()
-        self._check_pool_layout()
+        if fused_store:
+            self._check_pool_layout()
 
     def _check_pool_layout(self, layer_id: int = 0) -> None:
         """``forward`` writes new K/V rows into ``k_cache(layer)`` / ``v_cache(layer)`` itself (the key
@@ -649,6 +655,10 @@ class SharedCacheAttention:
         Hkv, D = self.num_kv_heads, self.head_dim
         key_pos = batch.positions if batch.mrope_positions is None else batch.mrope_positions
         key_pos = key_pos.to(device=self.device, dtype=torch.int64)
+        if not self.fused_store:
+            k_rot = self._rope(k.reshape(W, Hkv, D), key_pos)
+            self.kv_cache.store_kv(k_rot.view(W, Hkv * D), v.reshape(W, Hkv * D), batch.out_loc, layer_id)
+            return
         axis_stride = 0
         if key_pos.dim() == 2:
             key_pos = key_pos.contiguous()

@@ -81,3 +81,43 @@ def test_store_skips_negative_slots_and_touches_nothing_else(index_dtype, dtype)
                 expected[slot + 2, 0] = key[row]
                 expected[slot + 2, 1] = value[row]
         assert torch.equal(backing, expected)
+
+
+def test_new_rows_can_go_through_the_pools_own_store_kv():
+    """``fused_store=False``: the op rotates the new keys and hands K and V to ``kv_cache.store_kv`` as the
+    reference does (``attention.py:645-649``) instead of writing the pool itself -- for pools whose
+    ``store_kv`` does more than copy rows.  Same pool contents, same attention result, and the pool's method
+    is what ran."""
+    from types import SimpleNamespace
+
+    from async_llm_amd import workloads
+    from async_llm_amd.shared_cache import SharedCacheAttention
+
+    dev = torch.device("cuda")
+    wl = workloads.batched_decode(dev, workers=5, shared_len=300, private_lo=20, private_hi=200, heads=(8, 2, 64))
+    op = wl.op
+    want = op.forward(wl.q, wl.k, wl.v, 0, wl.batch)
+    want_k = wl.pool.k_cache(0).clone()
+    want_v = wl.pool.v_cache(0).clone()
+    # a second pool, same contents before the step, whose store_kv counts its calls
+    calls = []
+    k2, v2 = wl.pool.k_cache(0).clone(), wl.pool.v_cache(0).clone()
+    slots = wl.new_token_slots.long()
+    k2.view(-1, k2.shape[-2] * k2.shape[-1])[slots] = 0
+    v2.view(-1, v2.shape[-2] * v2.shape[-1])[slots] = 0
+
+    def store_kv(k, v, out_loc, layer_id):
+        calls.append(layer_id)
+        k2.view(-1, k.shape[-1])[out_loc.long()] = k
+        v2.view(-1, v.shape[-1])[out_loc.long()] = v
+
+    pool = SimpleNamespace(k_cache=lambda layer: k2, v_cache=lambda layer: v2, store_kv=store_kv)
+    other = SharedCacheAttention(pool, op.cos_sin_cache, op.num_qo_heads, op.num_kv_heads, op.head_dim, op.page_size,
+                                 op.dtype, dev, rotary_dim=op.rotary_dim, fused_store=False)
+    meta = other.prepare(wl.group, wl.pending, wl.new_token_slots)
+    batch = SimpleNamespace(attn_metadata=meta, positions=wl.batch.positions, out_loc=wl.batch.out_loc, mrope_positions=None)
+    got = other.forward(wl.q, wl.k, wl.v, 0, batch)
+    torch.cuda.synchronize()
+    assert calls == [0]
+    assert torch.equal(k2, want_k) and torch.equal(v2, want_v)
+    assert torch.equal(got, want)
