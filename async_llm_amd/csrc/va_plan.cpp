@@ -133,10 +133,10 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     }
   };
   std::vector<std::pair<int32_t, int32_t>> tiles;
-  // Decode groups (readers of one shared block) use wide tiles only on request: at decode sizes the
-  // extra launch costs more than the re-reads it saves; their narrow tiles are emitted chunk-major
-  // instead, so the tiles that stream the same chunk run side by side and share it in L2.
-  const bool wide_groups = params && params->wide_tile > 0;
+  // Decode groups (readers of one shared block): whether a group is cut into wide tiles is decided per
+  // group once the groups are known (group_is_wide below); narrow tiles are emitted chunk-major, so the
+  // tiles that stream the same chunk run side by side and share it in L2.
+  const bool wide_on_request = params && params->wide_tile > 0;
   const int target = params && params->target_items > 0 ? params->target_items
                                                         : std::max(64, 2048 / shape->num_kv_heads);
   const int gran = 64;  // chunk boundaries are multiples of this many tokens
@@ -186,6 +186,31 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
     }
   }
 
+  // Wide tiles for a group.  n readers in narrow tiles stream their block ceil(n / q_tile) times (once
+  // from memory, then from the die's L2), in wide tiles wide_tile / q_tile times less often -- but wide
+  // tiles run in a launch of their own, whose workgroups each stage a whole tile of queries and write a
+  // whole tile of partial states.  Measured at 16 q / 4 kv heads, head_dim 256, bf16 (q_tile 4, wide_tile
+  // 32 readers): 64 readers of an 8192-token block save 0.47 GB of such re-reads and the launch costs what
+  // they cost (401 -> 403 us); 128 readers of it save 0.94 GB (797 -> 759 us), 64 readers of a 32768-token
+  // block 1.9 GB (494 -> 443 us).  So: on request always; otherwise (plans of free size only) when the
+  // groups that would each save a fair share together save more than 0.64 GB.
+  std::vector<char> group_is_wide(groups.size(), wide_on_request && wide_tile > 0);
+  if (!wide_on_request && wide_tile > 0 && !cap) {
+    const int64_t token_bytes = 2ll * shape->num_kv_heads * shape->head_dim * (shape->dtype == VA_F32 ? 4 : 2);
+    constexpr int64_t kWorthALaunch = 640ll << 20, kFairShare = kWorthALaunch / 8;
+    std::vector<int64_t> saved(groups.size(), 0);
+    int64_t total = 0;
+    for (size_t gi = 0; gi < groups.size(); ++gi) {
+      const int64_t n = (int64_t)groups[gi].subrows.size();
+      if (n <= q_tile) continue;
+      cut_tiles(n, tiles, true);
+      saved[gi] = ((n + q_tile - 1) / q_tile - (int64_t)tiles.size()) * s->seq_lens[groups[gi].rep] * token_bytes;
+      if (saved[gi] >= kFairShare) total += saved[gi];
+    }
+    if (total >= kWorthALaunch)
+      for (size_t gi = 0; gi < groups.size(); ++gi) group_is_wide[gi] = saved[gi] >= kFairShare;
+  }
+
   // ---- chains: sub-requests of one prefill request, in table order ----
   std::vector<std::vector<int32_t>> chains;
   {
@@ -215,7 +240,7 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   // ---- total tokens -> chunk size for split-KV ----
   int64_t total_tokens = 0;
   for (auto& gr : groups) {
-    cut_tiles((int64_t)gr.subrows.size(), tiles, wide_groups);
+    cut_tiles((int64_t)gr.subrows.size(), tiles, group_is_wide[&gr - &groups[0]]);
     total_tokens += (int64_t)tiles.size() * s->seq_lens[gr.rep];
   }
   int64_t chain_tiles = 0, chain_tokens = 0, wide_chain_tokens = 0;
@@ -275,7 +300,7 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   // runs are cut finer: enough chunks for about one workgroup per CU.
   int64_t wide_group_tokens = 0;
   for (auto& gr : groups) {
-    cut_tiles((int64_t)gr.subrows.size(), tiles, wide_groups);
+    cut_tiles((int64_t)gr.subrows.size(), tiles, group_is_wide[&gr - &groups[0]]);
     for (auto& tl : tiles)
       if (tl.second - tl.first > q_tile) wide_group_tokens += s->seq_lens[gr.rep];
   }
@@ -286,7 +311,7 @@ int build(const VaSubRequests* s, const VaShape* shape, const VaPlanParams* para
   for (auto& gr : groups) {
     const int32_t rep = gr.rep;
     const int32_t len = s->seq_lens[rep];
-    cut_tiles((int64_t)gr.subrows.size(), tiles, wide_groups);
+    cut_tiles((int64_t)gr.subrows.size(), tiles, group_is_wide[&gr - &groups[0]]);
     // A run that a single query tile reads is fetched once per kv head and never again: its rows are
     // requested as lines to evict first, so that they stream through the die's L2 without pushing
     // out the rows that several tiles read side by side (a block shared by many views).

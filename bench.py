@@ -51,11 +51,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # carried here together with the digest of the kernel sources they were measured on
 # (csrc_digest()), and are reported only while that digest is the one of the sources in the tree.
 MEASURED_TRAFFIC = {
-    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_130_058 + 8_988) + 1024 * (17_882 + 512), "csrc": "883a29ab9aa0f9eb"},
-    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_098_017 + 4_722) + 1024 * (9_297 + 64), "csrc": "883a29ab9aa0f9eb"},
-    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_651_391 + 1024 * 131_526, "csrc": "883a29ab9aa0f9eb"},
-    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (440_240 + 1_623_106 + 27_058) + 1024 * (47_439 + 12_397 + 10_624),
-                              "csrc": "883a29ab9aa0f9eb"},
+    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_129_940 + 8_988) + 1024 * (17_883 + 512), "csrc": "14473b225f32621e"},
+    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_098_017 + 4_722) + 1024 * (9_297 + 64), "csrc": "14473b225f32621e"},
+    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_674_812 + 1024 * 131_520, "csrc": "14473b225f32621e"},
+    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (440_558 + 1_623_108 + 27_059) + 1024 * (47_441 + 12_398 + 10_624),
+                              "csrc": "14473b225f32621e"},
 }
 
 

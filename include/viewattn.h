@@ -147,7 +147,9 @@ typedef struct VaPlanParams {
   int32_t q_tile;        /* 0 = library default for the chosen kernel         */
   int32_t kv_chunk;      /* 0 = derive from the launch's total KV tokens      */
   int32_t target_items;  /* 0 = default (work items wanted per kv head)       */
-  int32_t wide_tile;     /* rows of a wide query tile: 0 = default, <0 = never */
+  int32_t wide_tile;     /* rows of a wide query tile: 0 = default (prefill tiles; decode readers of one
+                            block only where the re-reads saved outweigh a second launch), >0 = this many
+                            rows, decode readers included, <0 = never */
 } VaPlanParams;
 
 typedef struct VaPlanCounts {

@@ -176,6 +176,29 @@ def test_scaled_batched_and_mrope_configurations(kernel):
         assert wl.alg_bytes > 0 and wl.logical_bytes > 0
 
 
+@pytest.mark.parametrize("heads,readers", [((16, 4, 256), 40), ((8, 8, 128), 70), ((16, 2, 64), 21)])
+def test_many_readers_of_one_block_in_wide_tiles(heads, readers, monkeypatch):
+    """Decode readers of one block through the wide matrix-core kernel (tiles of 128 or 256 MFMA rows, taken
+    here on request; the planner takes them by itself only for blocks far too long for an oracle run), the
+    private blocks and the leftover readers through the streaming kernel, all merged per row."""
+    monkeypatch.setenv("VIEWATTN_PLAN", "wide_tile=%d" % (128 // (heads[0] // heads[1]) if heads[2] == 256 else
+                                                           256 // (heads[0] // heads[1])))
+    page = 16
+    op, cpu_pool, dev_pool, gen = make_op_and_pool(DEV, torch.bfloat16, heads, page, 1400, 1e7, seed=11, scale=1.0,
+                                                   kernel="auto", max_pos=8192)
+    pages = Pages(page)
+    shared = pages.block(1999)
+    views, targets = [], []
+    for w in range(readers):
+        mine = pages.block(5 + 23 * (w % 9))
+        views.append([shared, mine] if w % 5 else [mine, shared])
+        targets.append(mine)
+    *_, meta = run_decode_parity(op, cpu_pool, dev_pool, WorkerGroup(cache_structure=views, write_to=targets), pages,
+                                 1e7, gen, scale=1.0)
+    counts = meta.launch.counts
+    assert counts.n_wide_items > 0 and counts.n_items > counts.n_wide_items
+
+
 def test_forward_rejects_cpu_tensors_and_small_workspace():
     from async_llm_amd import native
 

@@ -41,6 +41,18 @@ def test_batched_decode_full_size_counts_every_token_once():
     assert torch.allclose(lse.double().cpu(), want, atol=1e-5, rtol=0), (lse.double().cpu() - want).abs().max()
 
 
+def test_long_shared_block_goes_wide_by_itself_and_counts_every_token_once():
+    # 64 readers of a 32768-token block: narrow tiles would stream it 16 times, the planner cuts the readers
+    # into two wide tiles (a launch of their own) without being asked
+    wl = workloads.batched_decode(DEV, layers=1, shared_len=32768)
+    assert wl.meta.launch.counts.n_wide_items > 0
+    out, lse = _zero_keys_unit_values(wl)
+    assert torch.equal(out, torch.ones_like(out))
+    tokens = torch.tensor([sum(b.num_tokens for b in view) + 1 for view in wl.group.cache_structure], dtype=torch.float64)
+    want = tokens.log()[:, None].expand(-1, wl.op.num_qo_heads)
+    assert torch.allclose(lse.double().cpu(), want, atol=1e-5, rtol=0), (lse.double().cpu() - want).abs().max()
+
+
 def test_view_prefill_full_size_counts_every_visible_token_once():
     wl = workloads.view_prefill(DEV, layers=1)  # configuration 3: 8 x 2048 new tokens over ~42 k tokens of view each
     out, lse = _zero_keys_unit_values(wl)

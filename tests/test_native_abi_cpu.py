@@ -318,6 +318,45 @@ def test_runs_that_one_tile_reads_are_flagged_read_once():
     assert seen[True] >= 3 and seen[False] >= len(private_len)
 
 
+def _shared_block_plan(readers, shared_len, wide_tile=0):
+    """`readers` requests over one shared block plus a private block each (bf16, 16 q / 4 kv heads, head_dim 256)."""
+    page = 16
+    shared_pages = list(range(-(-shared_len // page)))
+    kvi, kvp, lens, sw = [], [0], [], []
+    next_page = len(shared_pages)
+    for w in range(readers):
+        kvi += shared_pages; kvp.append(len(kvi)); lens.append(shared_len); sw.append(w)
+        n = 300 + 37 * w
+        kvi += list(range(next_page, next_page + -(-n // page))); next_page += -(-n // page)
+        kvp.append(len(kvi)); lens.append(n); sw.append(w)
+    n_sub = len(lens)
+    tables = (list(range(n_sub + 1)), kvp, lens, [0] * n_sub, sw, readers)
+    rc, blob, counts = build_plan(tables[0], kvp, kvi, lens, [0] * n_sub, [-1] * n_sub, sw, readers, heads=(16, 4, 256),
+                                  page=page, dtype=native.VA_BF16, kernel=native.VA_KERNEL_MFMA, wide_tile=wide_tile)
+    assert rc == 0, native.lib.va_last_error()
+    return blob, counts, tables
+
+
+def test_many_readers_of_a_long_block_get_wide_tiles_without_being_asked():
+    """Narrow tiles (4 requests) stream a block once per tile; wide ones (32 requests) an eighth as often, in a
+    launch of their own.  The planner takes them by itself only where the re-reads saved outweigh that launch:
+    64 readers x 8192 tokens (14 re-reads of 32 MB) stay narrow, 64 x 32768 and 128 x 8192 go wide; private
+    blocks (one reader) never do, a request for no wide tiles is honoured, and every pair is still covered once."""
+    for readers, shared_len, want_wide in [(64, 8192, False), (64, 32768, True), (128, 8192, True), (3, 65536, False)]:
+        blob, counts, tables = _shared_block_plan(readers, shared_len)
+        h, items, links, *_ = decode_plan(blob)
+        assert (counts.n_wide_items > 0) == want_wide, (readers, shared_len, counts.n_wide_items)
+        for it in items:
+            if it[2] and it[5]:  # a wide item: more than 4 requests, all on the shared block
+                assert int(it[2]) > 4 and all(int(l[0]) in tables[1][0::2] for l in links[it[0]: it[0] + it[1]])
+        check_coverage(blob, *tables)
+    blob, counts, tables = _shared_block_plan(64, 32768, wide_tile=-1)
+    assert counts.n_wide_items == 0
+    blob, counts, tables = _shared_block_plan(64, 8192, wide_tile=32)  # and on request always
+    assert counts.n_wide_items > 0
+    check_coverage(blob, *tables)
+
+
 def test_plan_rejects_inconsistent_tables():
     ok = dict(qo=[0, 1], kvp=[0, 2], kvi=[3, 4], lens=[8], flags=[0], chain=[-1], sub_worker=[0], n_rows=1)
 
