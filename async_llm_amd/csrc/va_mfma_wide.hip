@@ -35,6 +35,7 @@
 namespace va {
 
 constexpr int kWideThreads = 256;
+constexpr float kWideRaise = 14.f;  // a tile maximum this far above the reference (log2 units) raises it
 constexpr int kWideWaves = 4;
 constexpr int kWideTokens = 32;  // tokens per K/V tile
 #ifndef VA_WIDE_BUFFERS
@@ -137,6 +138,9 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   const bool pow2_pages = (P & (P - 1)) == 0;
   const int p_shift = __builtin_ctz(P);  // t / P and t % P as shift and mask (power-of-two pages)
   const int row_bytes = (int)a.pool_row_stride * (int)sizeof(S);
+  // bytes of a page, for the offsets of plain tiles: such tiles need the figure to fit 32 bits
+  const bool page_fits = ((unsigned long long)(uint32_t)row_bytes << p_shift) <= 0xffffffffull;
+  const uint32_t page_bytes = (uint32_t)row_bytes << p_shift;
 
   // This lane's part of a wave-level load (64 lanes x 16 bytes land as one 1 KB run in LDS; which
   // piece of the pool a lane fetches is free).  Waves 0 and 1 load K halves, waves 2 and 3 V halves.
@@ -195,12 +199,21 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   const int part_base = item[VA_I_PART_BASE];
   const bool wave_active = (kWaveRows * wave) / G < n_q;  // the wave owns real rows
 
-  float m_ref[kB], m_tile[kB], l_run[kB];  // reference maximum (log2 units), last tile maximum, row sum
+  float m_ref[kB], m_rel[kB], l_run[kB];  // reference maximum (log2 units), last tile maximum above `base`, row sum
+  // The score products start from -base instead of from zero (and the staged query carries the softmax
+  // scale), so a product's result IS the exponent s * scale - m_ref: base is the row's reference, or 0
+  // while the row has none yet (a reference of -1e30 would swallow the scores).
+  float base[kB], raise_above[kB];  // raise_above = m_ref + kWideRaise - base: what a tile's maximum is tested against
+  va_f32x16 score_start[kB];
   va_f32x16 o[kB][kDimTiles];
 #pragma unroll
   for (int b = 0; b < kB; ++b) {
     m_ref[b] = kNegBig;
-    m_tile[b] = kNegBig;
+    m_rel[b] = kNegBig;
+    base[b] = 0.f;
+    raise_above[b] = kNegBig + kWideRaise;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) score_start[b][r] = 0.f;
     l_run[b] = 0.f;
 #pragma unroll
     for (int t = 0; t < kDimTiles; ++t)
@@ -218,7 +231,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     const int causal_base = link[VA_L_CAUSAL_BASE];
     const bool slots = lflags & VA_LINK_SLOTS;
     // a 16-token half tile lies inside one page only if the link starts on a 16-token boundary
-    const bool uniform_pages = !slots && pow2_pages && P >= 16 && (tok_begin % 16 == 0);
+    const bool uniform_pages = !slots && pow2_pages && page_fits && P >= 16 && (tok_begin % 16 == 0);
 
     const int t_stop = min(tok_end, causal_base + n_q);  // tokens any row of the tile sees
     const int t_last = t_stop - 1;
@@ -245,18 +258,24 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
                               wave_half * 16 * kRowBytes;
     // pool row of this wave's half of tile i (uniform pages, tile inside the visible range); read
     // through the constant address space so that the lookup stays a scalar load
+    // (as a byte offset: page x bytes of a page + row in the page x bytes of a row, a 32 x 32 -> 64 bit
+    // product and a 32-bit one; the row number times the row size would be a 64 x 32 bit product, six
+    // scalar instructions in every ring step)
+    auto half_offset = [&](int page, int t) __attribute__((always_inline)) {
+      return (unsigned long long)(uint32_t)page * page_bytes + (uint32_t)(t & (P - 1)) * (uint32_t)row_bytes;
+    };
     auto half_row = [&](int i) __attribute__((always_inline)) {
       const int t = tok_begin + i * kWideTokens + 16 * wave_half;
       const int page = ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + (t >> p_shift)];
-      return ((long long)page << p_shift) + (t & (P - 1));
+      return half_offset(page, t);
     };
     auto tile_is_plain = [&](int i) __attribute__((always_inline)) {
       return uniform_pages && tok_begin + (i + 1) * kWideTokens - 1 <= t_last;
     };
-    auto issue = [&](int i, long long row) __attribute__((always_inline)) {
+    auto issue = [&](int i, unsigned long long row) __attribute__((always_inline)) {
       const uint32_t dst = wave_lds + ring_slot(i) * Sh::kBufferBytes;
       if (tile_is_plain(i)) {
-        const char* base = wave_plain + row * row_bytes;
+        const char* base = wave_plain + row;
         issue_plain(base, dst);
       } else {
         const int t0 = tok_begin + i * kWideTokens + 16 * wave_half;
@@ -323,12 +342,12 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
 #pragma unroll
             for (int jj = 0; jj < kBatch; ++jj) unit[jj].load(a.rope, qh[jj], x, pos[jj]);
 #pragma unroll
-            for (int jj = 0; jj < kBatch; ++jj) unit[jj].finish(a.rope, pos[jj], p0[jj], p1[jj]);
+            for (int jj = 0; jj < kBatch; ++jj) unit[jj].finish(a.rope, pos[jj], p0[jj], p1[jj], a.scale_log2);
           } else {
 #pragma unroll
             for (int jj = 0; jj < kBatch; ++jj) {
-              p0[jj] = *(const uint4*)(qh[jj] + 8 * c0);
-              p1[jj] = *(const uint4*)(qh[jj] + 8 * c1);
+              p0[jj] = scaled_piece<E>(*(const uint4*)(qh[jj] + 8 * c0), a.scale_log2);
+              p1[jj] = scaled_piece<E>(*(const uint4*)(qh[jj] + 8 * c1), a.scale_log2);
             }
           }
 #pragma unroll
@@ -353,6 +372,8 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
             const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
             const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
             rotated_query_unit<E>(a.rope, qh, x, p, c0, c1, p0, p1);
+            p0 = scaled_piece<E>(p0, a.scale_log2);
+            p1 = scaled_piece<E>(p1, a.scale_log2);
           }
           q_stage[Rl * kChunks + (c0 ^ wide_swz<kD>(Rl))] = va_u32x4{p0.x, p0.y, p0.z, p0.w};
           q_stage[Rl * kChunks + (c1 ^ wide_swz<kD>(Rl))] = va_u32x4{p1.x, p1.y, p1.z, p1.w};
@@ -369,12 +390,15 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
 
     // ---- the tile loop ----
     // Reference maximum.  The softmax runs against a per-row REFERENCE maximum m_ref that is
-    // raised only when a tile's maximum exceeds it by more than kRaise (in log2 units):
-    // p = exp2(s - m_ref) then stays below 2^kRaise, harmless for the 16-bit P operand and the
+    // raised only when a tile's maximum exceeds it by more than kWideRaise (in log2 units):
+    // p = exp2(s - m_ref) then stays below 2^kWideRaise, harmless for the 16-bit P operand and the
     // fp32 sums, and any consistent reference gives the same softmax.  Raising m_ref means
     // rescaling the D fp32 accumulators of every row, vector-ALU work on registers that otherwise
     // only the matrix pipe touches; it happens on the first tile and then hardly ever, so it is
-    // kept out of the hot loop: the loop breaks, the accumulators are rescaled, the loop resumes.
+    // kept out of the hot loop: the steady loop is left, the accumulators are rescaled, the tile is
+    // computed, the steady loop is entered again.  (One wave per SIMD issues an instruction every four
+    // clocks or so whatever its kind: the steady loop's own control being a counter and one test,
+    // instead of the general loop's flags, is worth 2 % of the kernel.)
     //
     // Software pipeline.  One wave per SIMD means nothing but this wave's own instruction order
     // can keep the matrix pipe busy, so the loop body is written as pieces pinned in order with
@@ -386,19 +410,18 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     // request tile k + 2 into the buffer of tile k - 2, which every wave has left by then.  Every
     // wave makes every step exactly once, in order; a step is made just before tile k is first
     // needed (its K, for the scores computed one iteration ahead).
-    constexpr float kRaise = 14.f;
     const int n_vis = t_wave > tok_begin ? min(n_tiles, (t_wave - tok_begin + kWideTokens - 1) / kWideTokens) : 0;
     int next_step = 0;
     // The pool row of the tile a step requests is looked up a whole step earlier (a scalar load whose
     // result is not touched before the next step): its latency never shows.
     auto row_of = [&](int tile) __attribute__((always_inline)) {
-      return (tile < n_tiles && tile_is_plain(tile)) ? half_row(tile) : 0ll;
+      return (tile < n_tiles && tile_is_plain(tile)) ? half_row(tile) : 0ull;
     };
-    long long row_ahead = row_of(kWideAhead);
+    unsigned long long row_ahead = row_of(kWideAhead);
     auto ring_step = [&]() __attribute__((always_inline)) {
       const int k = next_step++;
       const bool refill = k + kWideAhead < n_tiles;
-      const long long row = row_ahead;
+      const unsigned long long row = row_ahead;
       row_ahead = row_of(k + 1 + kWideAhead);
       // only the loads of the tiles requested after tile k (up to kWideAhead - 1 of them) may still be outstanding
       if (k + kWideAhead - 1 < n_tiles) {
@@ -414,16 +437,19 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
     // The same step for the steady part of a link (uniform pages; the requested tile and the one
     // after it inside the visible range): no case distinctions, and the page lookup for the next
     // step is sent before the barrier and first touched after it, so its latency passes under the wait.
+    const __attribute__((address_space(4))) char* link_pages =
+        (const __attribute__((address_space(4))) char*)(a.kv_indices + kv_begin);
     auto ring_step_steady = [&]() __attribute__((always_inline)) {
       const int k = next_step++;
-      const long long row = row_ahead;
+      const unsigned long long row = row_ahead;
       const int t = tok_begin + (k + 1 + kWideAhead) * kWideTokens + 16 * wave_half;
-      const int page = ((const __attribute__((address_space(4))) int32_t*)a.kv_indices)[kv_begin + (t >> p_shift)];
+      // (base of the link's page list + an unsigned 32-bit byte offset: a scalar load with a register offset)
+      const int page = *(const __attribute__((address_space(4))) int32_t*)(link_pages + ((uint32_t)(t >> p_shift) << 2));
       const int zero = ring_barrier_zero<(kWideAhead - 1) * kL>();
       const uint32_t dst = wave_lds + ring_slot(k + kWideAhead) * Sh::kBufferBytes;
-      const char* base = wave_plain + row * row_bytes;
+      const char* base = wave_plain + row;
       issue_plain(base, dst);
-      row_ahead = ((long long)(page + zero) << p_shift) + (t & (P - 1));
+      row_ahead = half_offset(page + zero, t);
     };
     // iterations [1, i_steady_end) may take it: tiles i + 1 + kWideAhead and i + 2 + kWideAhead are plain,
     // tile i is unmasked for every row of the wave and a next tile exists
@@ -434,209 +460,220 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       i_steady_end = min(min(plain_tiles - 2 - kWideAhead, unmasked_tiles), n_vis - 1);
     }
 
-    va_f32x16 sc[kB];       // scores, then probabilities, of the current tile
-    va_f32x16 sc_next[kB];  // scores of the next tile, accumulating
-    va_u32x4 kf[kSteps];
-    auto read_k = [&](int tile) __attribute__((always_inline)) {
+    // Scores of two tiles: the exponentials of one are taken in place while the products of the next
+    // accumulate into the other; which is which alternates from tile to tile.
+    va_f32x16 sc[kB];       // scores, then probabilities, of the current tile (between tiles)
+    va_f32x16 sc_next[kB];  // scores of the next tile
+    // K fragments: at most eight in registers; the fragment eight steps on is requested as one is consumed
+    constexpr int kKRing = kSteps < 8 ? kSteps : 8;
+    va_u32x4 kf[kKRing];
+    auto read_k_fragment = [&](int tile, int s) __attribute__((always_inline)) {
       const char* kt = lds + ring_slot(tile) * Sh::kBufferBytes;
-#pragma unroll
-      for (int s = 0; s < kSteps; ++s) kf[s] = *(const va_u32x4*)(kt + k_lane_byte + 256 * s);
+      kf[s % kKRing] = *(const va_u32x4*)(kt + k_lane_byte + 256 * s);
     };
-    auto score_step = [&](int s) __attribute__((always_inline)) {
+    auto read_k = [&](int tile) __attribute__((always_inline)) {
+#pragma unroll
+      for (int s = 0; s < kKRing; ++s) read_k_fragment(tile, s);
+    };
+    auto score_step = [&](int tile, int s, auto& into) __attribute__((always_inline)) {
 #pragma unroll
       for (int b = 0; b < kB; ++b) {
         // through the builtin: the compiler sees these products and keeps the wait states between
         // them and the vector-ALU instructions that feed them or read their results
-        if (s == 0) {
-          sc_next[b] = Mma<E>::run32(kf[s], qf[b][s], va_f32x16{});
-        } else {
-          sc_next[b] = Mma<E>::run32(kf[s], qf[b][s], sc_next[b]);
-        }
+        into[b] = Mma<E>::run32(kf[s % kKRing], qf[b][s], s == 0 ? score_start[b] : into[b]);
       }
+      if (s + kKRing < kSteps) read_k_fragment(tile, s + kKRing);
     };
 
     if (n_vis > 0) {  // scores of tile 0
       ring_step();
       read_k(0);
 #pragma unroll
-      for (int s = 0; s < kSteps; ++s) score_step(s);
-#pragma unroll
-      for (int b = 0; b < kB; ++b) sc[b] = sc_next[b];
+      for (int s = 0; s < kSteps; ++s) score_step(0, s, sc);
     }
-    bool resume = false;  // the step for tile i + 1 is made and sc holds the (masked) scores of tile i
-    bool sc_is_raw = true;  // sc holds the raw scores of the first tile (no reference maximum exists yet)
     // maximum of the (unmasked) scores of the next tile per lane, gathered piecewise between the
     // P.V products of the current one, whose matrix work leaves the vector ALU idle
     float early_max[kB];
     bool early_max_valid = false;
 #pragma unroll
     for (int b = 0; b < kB; ++b) early_max[b] = 0.f;
-    int i = 0;
-    while (i < n_vis) {
-      for (; i < n_vis; ++i) {
-        const int t0 = tok_begin + i * kWideTokens;
-        const bool has_next = i + 1 < n_vis;
-        if (!resume && i >= 1 && i < i_steady_end) {
-          // steady part: the maxima were gathered under the previous products, nothing is masked
-          ring_step_steady();
-          bool raise = false;
+    // One tile: phase A and phase B below, on the scores in `cur`, leaving those of the next tile in `nxt`.
+    // The steady part of a link runs it in a loop of its own, whose control is a counter and the test for
+    // a raised reference; every other tile (the first, masked ones, the last, the one after a raised
+    // reference) goes through the general step further down.
+    auto tile_body = [&](int i, auto& cur, auto& nxt) __attribute__((always_inline)) {
+
+      // V^T fragments of this tile, kVAhead of them in flight: fragment idx = (step kk, dim tile t)
+      const uint32_t vt = lds_base + ring_slot(i) * Sh::kBufferBytes + Sh::kTileBytes;
+      const uint32_t vt_even = vt + v_even, vt_odd = vt + v_odd;
+      constexpr int kFrags = 2 * kDimTiles;
+      constexpr int kMaxFirst = kFrags > 2 ? 2 : kFrags - 1;  // first product the early maxima follow
+      constexpr int kVAhead = kFrags < 4 ? kFrags : 4;
+      va_u32x4 vfr[kVAhead];
+      auto read_vfrag = [&](int idx) __attribute__((always_inline)) {
+        const int kk = idx / kDimTiles, t = idx % kDimTiles;
+        const uint32_t at = ((t & 1) ? vt_odd : vt_even) + 128 * (t / 2) + kk * 16 * kRowBytes;
+        const va_u32x2 lo = lds_read_tr16(at), hi = lds_read_tr16(at + 8 * kRowBytes);
+        vfr[idx % kVAhead] = va_u32x4{lo[0], lo[1], hi[0], hi[1]};
+      };
+      // ---- phase A: scores of tile i + 1 (matrix pipe) under the exponentials of tile i ----
+      float sum[kB];
 #pragma unroll
-          for (int b = 0; b < kB; ++b) {
-            m_tile[b] = half_wave_max(early_max[b] * a.scale_log2);
-            raise = raise || m_tile[b] > m_ref[b] + kRaise;
-          }
-          if (__any(raise)) {
-            resume = true;
-            break;
-          }
-        } else if (!resume) {
-          if (i + 1 < n_tiles) ring_step();  // tile i + 1 has landed
-          // mask and find the tile maxima; reg r of a block is token t0 + (r/4)*8 + 4h + r%4 of its row
-          const bool masked = t0 + kWideTokens > t_wave_min;
-          bool raise = false;
+      for (int b = 0; b < kB; ++b) sum[b] = 0.f;
+      // Piece r: the exponential of element r; the sum takes element r - 1 (an exponential's result
+      // is not ready for the very next instruction) and odd pieces pack the finished pair into P.
+      uint32_t pw[kB][8];
+      auto exp_piece = [&](int r) __attribute__((always_inline)) {
 #pragma unroll
-          for (int b = 0; b < kB; ++b) {
-            if (masked) {
+        for (int b = 0; b < kB; ++b) {
+          cur[b][r] = __builtin_amdgcn_exp2f(cur[b][r]);  // the scores came out of their products as s * scale - m_ref
+          if (r > 0) sum[b] += cur[b][r - 1];
+          if (r >= 2 && r % 2 == 0) pw[b][r / 2 - 1] = Mma<E>::pack(cur[b][r - 2], cur[b][r - 1]);
+        }
+      };
+      constexpr int kPiecesPerStep = 16 / kSteps > 0 ? 16 / kSteps : 1;  // exponentials between two score steps
+      // The last visible tile runs the same instructions: its "next scores" come from whatever
+      // the following ring buffer holds and are never looked at (sixteen idle products per link
+      // against a second copy of this phase and the register moves where the two would meet).
+      read_k(i + 1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-              for (int r = 0; r < 16; ++r)
-                sc[b][r] = (t0 + (r / 4) * 8 + 4 * h + (r % 4)) < t_row[b] ? sc[b][r] : -INFINITY;
-            }
-            // the tile maximum in log2 units: from the raw maxima found under the previous products, or,
-            // for a masked or first tile, from sc (raw scores on the first tile, else already s - m_ref)
-            float tile_max = early_max[b] * a.scale_log2;
-            if (masked || !early_max_valid) {
-              tile_max = sc[b][0];
+      for (int r = 0; r < 16; ++r) {
+        if (r % kPiecesPerStep == 0) score_step(i + 1, r / kPiecesPerStep, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        exp_piece(r);
+        // the first V fragments are requested once half of the K fragments have been consumed: the
+        // counter of outstanding LDS reads holds fifteen, and a wait for the first K fragment
+        // with more than that in flight becomes a wait for the excess as well
+        if (r == 8) {
 #pragma unroll
-              for (int r = 1; r < 16; ++r) tile_max = fmaxf(tile_max, sc[b][r]);
-              tile_max = sc_is_raw ? tile_max * a.scale_log2 : tile_max + m_ref[b];
-            }
-            m_tile[b] = half_wave_max(tile_max);
-            raise = raise || m_tile[b] > m_ref[b] + kRaise;
-          }
-          if (__any(raise) || sc_is_raw) {  // the first tile always sets the references
-            resume = true;
-            break;
+          for (int idx = 0; idx < kVAhead; ++idx) read_vfrag(idx);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int b = 0; b < kB; ++b) {
+        l_run[b] += sum[b] + cur[b][15];
+        pw[b][7] = Mma<E>::pack(cur[b][14], cur[b][15]);
+      }
+
+      // ---- phase B: O^T += V^T . P^T over two 16-token steps; a fragment serves all row blocks,
+      // and once it has been used the fragment kVAhead further on is requested ----
+      va_u32x4 pf[2][kB];
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int b = 0; b < kB; ++b)
+          pf[kk][b] = va_u32x4{pw[b][4 * kk + 0], pw[b][4 * kk + 1], pw[b][4 * kk + 2], pw[b][4 * kk + 3]};
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int idx = 0; idx < kFrags; ++idx) {
+        const int kk = idx / kDimTiles, t = idx % kDimTiles;
+#pragma unroll
+        for (int b = 0; b < kB; ++b) {
+          Mma<E>::run32_acc(vfr[idx % kVAhead], pf[kk][b], o[b][t]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (idx + kVAhead < kFrags) read_vfrag(idx + kVAhead);
+        // Elements of the next tile's scores folded into early_max after this product: the 15
+        // comparisons are spread over the products from the third on (the last score product was
+        // issued well before, so its results have been written).
+        if (idx >= kMaxFirst) {
+#pragma unroll
+          for (int e = 1; e < 16; ++e) {
+            if (kMaxFirst + (e - 1) * (kFrags - kMaxFirst) / 15 != idx) continue;
+#pragma unroll
+            for (int b = 0; b < kB; ++b)
+              early_max[b] = fmaxf(e == 1 ? nxt[b][0] : early_max[b], nxt[b][e]);
           }
         }
-        resume = false;
-
-        // V^T fragments of this tile, kVAhead of them in flight: fragment idx = (step kk, dim tile t)
-        const uint32_t vt = lds_base + ring_slot(i) * Sh::kBufferBytes + Sh::kTileBytes;
-        const uint32_t vt_even = vt + v_even, vt_odd = vt + v_odd;
-        constexpr int kFrags = 2 * kDimTiles;
-        constexpr int kMaxFirst = kFrags > 2 ? 2 : kFrags - 1;  // first product the early maxima follow
-        constexpr int kVAhead = kFrags < 4 ? kFrags : 4;
-        va_u32x4 vfr[kVAhead];
-        auto read_vfrag = [&](int idx) __attribute__((always_inline)) {
-          const int kk = idx / kDimTiles, t = idx % kDimTiles;
-          const uint32_t at = ((t & 1) ? vt_odd : vt_even) + 128 * (t / 2) + kk * 16 * kRowBytes;
-          const va_u32x2 lo = lds_read_tr16(at), hi = lds_read_tr16(at + 8 * kRowBytes);
-          vfr[idx % kVAhead] = va_u32x4{lo[0], lo[1], hi[0], hi[1]};
-        };
-        // ---- phase A: scores of tile i + 1 (matrix pipe) under the exponentials of tile i ----
-        float sum[kB];
-#pragma unroll
-        for (int b = 0; b < kB; ++b) sum[b] = 0.f;
-        // Piece r: the exponential of element r; the sum takes element r - 1 (an exponential's result
-        // is not ready for the very next instruction) and odd pieces pack the finished pair into P.
-        uint32_t pw[kB][8];
-        auto exp_piece = [&](int r) __attribute__((always_inline)) {
-#pragma unroll
-          for (int b = 0; b < kB; ++b) {
-            sc[b][r] = __builtin_amdgcn_exp2f(sc[b][r]);  // sc holds s - m_ref already
-            if (r > 0) sum[b] += sc[b][r - 1];
-            if (r >= 2 && r % 2 == 0) pw[b][r / 2 - 1] = Mma<E>::pack(sc[b][r - 2], sc[b][r - 1]);
-          }
-        };
-        constexpr int kPiecesPerStep = 16 / kSteps > 0 ? 16 / kSteps : 1;  // exponentials between two score steps
-        // The last visible tile runs the same instructions: its "next scores" come from whatever
-        // the following ring buffer holds and are never looked at (sixteen idle products per link
-        // against a second copy of this phase and the register moves where the two would meet).
-        read_k(i + 1);
         __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // The reference of the rows is raised to the maxima of the tile in `cur` (m_rel, above base): what was
+    // accumulated against the old reference is rescaled, and so are the tile's scores; the products that
+    // follow start from the new one.
+    auto raise_reference = [&](int i, auto& cur) __attribute__((always_inline)) {
+      accumulator_fence<kB * kDimTiles>(&o[0][0]);
+#pragma unroll
+      for (int b = 0; b < kB; ++b) {
+        const float m_new = fmaxf(m_ref[b], m_rel[b] + base[b]);
+        const float alpha = __builtin_amdgcn_exp2f(m_ref[b] - m_new);
+        const float step = m_new - base[b];
+        m_ref[b] = m_new;
+        l_run[b] *= alpha;
+#pragma unroll
+        for (int t = 0; t < kDimTiles; ++t) o[b][t] *= alpha;
+        const int t0 = tok_begin + i * kWideTokens;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          if (r % kPiecesPerStep == 0) score_step(r / kPiecesPerStep);
-          __builtin_amdgcn_sched_barrier(0);
-          exp_piece(r);
-          // the first V fragments are requested once half of the K fragments have been consumed: the
-          // counter of outstanding LDS reads holds fifteen, and a wait for the first K fragment
-          // with more than that in flight becomes a wait for the excess as well
-          if (r == 8) {
-#pragma unroll
-            for (int idx = 0; idx < kVAhead; ++idx) read_vfrag(idx);
-          }
-          __builtin_amdgcn_sched_barrier(0);
+          const bool visible = (t0 + (r / 4) * 8 + 4 * h + (r % 4)) < t_row[b];
+          cur[b][r] = visible ? cur[b][r] - step : -INFINITY;
         }
+        base[b] = m_new > 0.5f * kNegBig ? m_new : 0.f;  // (a row that has seen nothing yet keeps base 0)
+        raise_above[b] = m_new + kWideRaise - base[b];
 #pragma unroll
-        for (int b = 0; b < kB; ++b) {
-          l_run[b] += sum[b] + sc[b][15];
-          pw[b][7] = Mma<E>::pack(sc[b][14], sc[b][15]);
-        }
+        for (int r = 0; r < 16; ++r) score_start[b][r] = -base[b];
+      }
+    };
+    // the test of the steady part: the maxima were gathered under the previous products, nothing is masked
+    auto steady_test = [&]() __attribute__((always_inline)) {
+      bool raise = false;
+#pragma unroll
+      for (int b = 0; b < kB; ++b) {
+        m_rel[b] = half_wave_max(early_max[b]);
+        raise = raise || m_rel[b] > raise_above[b];
+      }
+      return (bool)__any(raise);
+    };
 
-        // ---- phase B: O^T += V^T . P^T over two 16-token steps; a fragment serves all row blocks,
-        // and once it has been used the fragment kVAhead further on is requested ----
-        va_u32x4 pf[2][kB];
+    int i = 0;
+    while (i < n_vis) {
+      bool raise = false;
+      if (i >= 1 && i < i_steady_end) {
+        // steady part
+        do {
+          ring_step_steady();
+          raise = steady_test();
+          if (raise) break;
+          tile_body(i, sc, sc_next);
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-          for (int b = 0; b < kB; ++b)
-            pf[kk][b] = va_u32x4{pw[b][4 * kk + 0], pw[b][4 * kk + 1], pw[b][4 * kk + 2], pw[b][4 * kk + 3]};
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int idx = 0; idx < kFrags; ++idx) {
-          const int kk = idx / kDimTiles, t = idx % kDimTiles;
-#pragma unroll
-          for (int b = 0; b < kB; ++b) {
-            Mma<E>::run32_acc(vfr[idx % kVAhead], pf[kk][b], o[b][t]);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-          if (idx + kVAhead < kFrags) read_vfrag(idx + kVAhead);
-          // Elements of the next tile's scores folded into early_max after this product: the 15
-          // comparisons are spread over the products from the third on (the last score product was
-          // issued well before, so its results have been written).
-          if (idx >= kMaxFirst) {
-#pragma unroll
-            for (int e = 1; e < 16; ++e) {
-              if (kMaxFirst + (e - 1) * (kFrags - kMaxFirst) / 15 != idx) continue;
-#pragma unroll
-              for (int b = 0; b < kB; ++b)
-                early_max[b] = fmaxf(e == 1 ? sc_next[b][0] : early_max[b], sc_next[b][e]);
-            }
-            // ... and moved to sc as s * scale - m_ref, what the exponentials of the next iteration
-            // start from (P of this tile has left sc; a raised reference redoes this from sc_next)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-              if (kMaxFirst + e * (kFrags - kMaxFirst) / 16 != idx) continue;
-#pragma unroll
-              for (int b = 0; b < kB; ++b) sc[b][e] = fmaf(sc_next[b][e], a.scale_log2, -m_ref[b]);
-            }
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        early_max_valid = has_next;
-      }
-      if (resume) {
-        // raise the references to this tile's maxima and rescale what was accumulated against the old ones
-        accumulator_fence<kB * kDimTiles>(&o[0][0]);
+          for (int b = 0; b < kB; ++b) sc[b] = sc_next[b];
+          ++i;
+        } while (i < i_steady_end);
+        early_max_valid = true;  // (a next tile exists throughout the steady part)
+        if (!raise) continue;
+      } else {
+        const int t0 = tok_begin + i * kWideTokens;
+        if (i + 1 < n_tiles) ring_step();  // tile i + 1 has landed
+        // mask and find the tile maxima; reg r of a block is token t0 + (r/4)*8 + 4h + r%4 of its row
+        const bool masked = t0 + kWideTokens > t_wave_min;
 #pragma unroll
         for (int b = 0; b < kB; ++b) {
-          const float m_new = fmaxf(m_ref[b], m_tile[b]);
-          const float alpha = __builtin_amdgcn_exp2f(m_ref[b] - m_new);
-          m_ref[b] = m_new;
-          l_run[b] *= alpha;
+          if (masked) {
 #pragma unroll
-          for (int t = 0; t < kDimTiles; ++t) o[b][t] *= alpha;
-          // sc_next still holds this tile's raw scores: sc = s * scale - m_ref against the new reference
-          const int t0 = tok_begin + i * kWideTokens;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const bool visible = (t0 + (r / 4) * 8 + 4 * h + (r % 4)) < t_row[b];
-            sc[b][r] = visible ? fmaf(sc_next[b][r], a.scale_log2, -m_ref[b]) : -INFINITY;
+            for (int r = 0; r < 16; ++r)
+              sc[b][r] = (t0 + (r / 4) * 8 + 4 * h + (r % 4)) < t_row[b] ? sc[b][r] : -INFINITY;
           }
+          // the tile maximum above base: from the maxima found under the previous products, or, for a
+          // masked or first tile, from sc
+          float tile_max = early_max[b];
+          if (masked || !early_max_valid) {
+            tile_max = sc[b][0];
+#pragma unroll
+            for (int r = 1; r < 16; ++r) tile_max = fmaxf(tile_max, sc[b][r]);
+          }
+          m_rel[b] = half_wave_max(tile_max);
+          raise = raise || m_rel[b] > raise_above[b];
         }
-        sc_is_raw = false;
+        raise = __any(raise);
       }
+      if (raise) raise_reference(i, sc);
+      tile_body(i, sc, sc_next);
+#pragma unroll
+      for (int b = 0; b < kB; ++b) sc[b] = sc_next[b];
+      early_max_valid = i + 1 < n_vis;
+      ++i;
     }
     while (next_step < n_tiles) ring_step();  // tiles this wave does not see: keep in step with the others
   }
