@@ -271,3 +271,45 @@ def test_wide_tiles_with_a_late_score_spike(D, dtype, spike):
         # dim, so the spike's exponent is off by up to 2^-8 of itself in bf16 (2^-11 in fp16).
         staged = spike * 0.6931 * 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
         assert torch.allclose(got, want[:, None].expand_as(got), atol=2e-2 + staged, rtol=0)
+
+
+@pytest.mark.parametrize("spike", [15.0, 60.0])
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 256), (torch.float16, 128), (torch.bfloat16, 64)])
+def test_wide_tiles_with_a_spike_in_the_first_tile_of_a_later_block(D, dtype, spike):
+    """The reference maximum of a row is carried from block to block of a view (the score products of a tile
+    start from minus that reference).  Here the first context block holds zero keys only, so the reference
+    settles at 0, and the SECOND block opens with a key whose score is ``spike`` log2 units for every row: the
+    raise happens on the first tile of a link, where no maxima were gathered ahead.  A third block of zero keys
+    follows (scores far below the raised reference).  Closed form: every other score is 0."""
+    heads, page, rotary = (8, 2, D), 16, D // 2
+    op, cpu_pool, dev_pool, gen = make_op_and_pool(DEV, dtype, heads, page, 128, 1e4, rotary_dim=rotary, seed=17,
+                                                   scale=1.0, kernel="auto", max_pos=4096)
+    a = spike * 2.0 / (D ** 0.5 * 1.4426950408889634)
+    for pool in (cpu_pool[0], dev_pool[0]):
+        pool.zero_()
+    blocks, first_page = [], 0
+    for n in (256, 300, 130):
+        b = CacheBlock(DEV, page)
+        b.grow_pages(torch.arange(first_page, first_page + -(-n // page)) * page, n)
+        first_page += -(-n // page)
+        blocks.append(b)
+    planted = (256 // page) * page + 3  # token 3 of the second block (pages are in order here)
+    for pool in (cpu_pool[0], dev_pool[0]):
+        pool.view(-1, heads[1], D)[planted, :, rotary:] = a
+    new_tokens, prefix = 160, 16
+    pages = torch.arange(60, 60 + -(-(prefix + new_tokens) // page), dtype=torch.int32) * page
+    specs = [PrefillSpec(blocks, pages, new_tokens, prefix)]
+
+    def mutate(q, k, v):
+        q.view(-1, heads[0], D)[:, :, rotary:] = 1.0
+        k.zero_()
+
+    out, lse, exp_out, exp_lse, meta = run_prefill_parity(op, cpu_pool, dev_pool, specs, 1e4, gen, scale=1.0,
+                                                          mutate=mutate)
+    assert meta.launch.counts.n_wide_items > 0
+    seen = 256 + 300 + 130 + prefix + torch.arange(1, new_tokens + 1, dtype=torch.float64)
+    a_stored = float(torch.tensor(a, dtype=dtype))
+    want = (seen - 1 + torch.tensor(a_stored * (D / 2) / D ** 0.5, dtype=torch.float64).exp()).log()
+    got = lse.double().cpu()
+    staged = spike * 0.6931 * 2.0 ** (-8 if dtype == torch.bfloat16 else -11)  # (the staged query's rounding, see above)
+    assert torch.allclose(got, want[:, None].expand_as(got), atol=2e-2 + staged, rtol=0)
