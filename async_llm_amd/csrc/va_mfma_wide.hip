@@ -445,10 +445,20 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       const int t = tok_begin + (k + 1 + kWideAhead) * kWideTokens + 16 * wave_half;
       // (base of the link's page list + an unsigned 32-bit byte offset: a scalar load with a register offset)
       const int page = *(const __attribute__((address_space(4))) int32_t*)(link_pages + ((uint32_t)(t >> p_shift) << 2));
-      const int zero = ring_barrier_zero<(kWideAhead - 1) * kL>();
+      // The K half of the buffer refilled here was last read two steps ago (the scores of a tile are computed
+      // an iteration ahead of its products), and every wave has passed a barrier since: the waves that load K
+      // send their requests BEFORE the barrier, in the time they would otherwise only wait, and out of step
+      // with the waves that load V, which must wait for the products of the previous iteration to end.
+      int zero;
       const uint32_t dst = wave_lds + ring_slot(k + kWideAhead) * Sh::kBufferBytes;
       const char* base = wave_plain + row;
-      issue_plain(base, dst);
+      if (!wave_is_v) {
+        issue_plain(base, dst);
+        zero = ring_barrier_zero<kWideAhead * kL>();
+      } else {
+        zero = ring_barrier_zero<(kWideAhead - 1) * kL>();
+        issue_plain(base, dst);
+      }
       row_ahead = half_offset(page + zero, t);
     };
     // iterations [1, i_steady_end) may take it: tiles i + 1 + kWideAhead and i + 2 + kWideAhead are plain,
