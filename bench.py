@@ -51,11 +51,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # carried here together with the digest of the kernel sources they were measured on
 # (csrc_digest()), and are reported only while that digest is the one of the sources in the tree.
 MEASURED_TRAFFIC = {
-    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_129_637 + 8_988) + 1024 * (17_885 + 512), "csrc": "54a734d96c9153d1"},
-    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_098_018 + 4_722) + 1024 * (9_297 + 64), "csrc": "54a734d96c9153d1"},
-    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_569_445 + 1024 * 131_916, "csrc": "54a734d96c9153d1"},
-    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (440_095 + 1_623_107 + 27_058) + 1024 * (47_440 + 12_397 + 10_624),
-                              "csrc": "54a734d96c9153d1"},
+    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_130_005 + 8_988) + 1024 * (17_883 + 512), "csrc": "778986fa809c6eea"},
+    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_098_018 + 4_722) + 1024 * (9_297 + 64), "csrc": "778986fa809c6eea"},
+    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_510_557 + 1024 * 131_393, "csrc": "778986fa809c6eea"},
+    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (439_625 + 1_623_110 + 27_059) + 1024 * (47_445 + 12_397 + 10_624),
+                              "csrc": "778986fa809c6eea"},
 }
 
 
