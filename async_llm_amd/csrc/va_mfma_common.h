@@ -176,10 +176,7 @@ struct TableQueryUnit {
     s[0] = *(const float4*)(row + rope.half);
     s[1] = *(const float4*)(row + rope.half + 4);
   }
-  // `qs`: a factor the rotated values carry into their one rounding (the wide kernel stages the query
-  // times the softmax scale, so that its score products come out as exponents)
-  __device__ __forceinline__ void finish(const RopeDev& rope, const Pos3& p, uint4& o0, uint4& o1,
-                                         float qs = 1.f) const {
+  __device__ __forceinline__ void finish(const RopeDev& rope, const Pos3& p, uint4& o0, uint4& o1) const {
     using S = typename E::storage;
     const uint32_t wa[4] = {ra.x, ra.y, ra.z, ra.w}, wb[4] = {rb.x, rb.y, rb.z, rb.w};
     const float ct[8] = {c[0].x, c[0].y, c[0].z, c[0].w, c[1].x, c[1].y, c[1].z, c[1].w};
@@ -197,28 +194,13 @@ struct TableQueryUnit {
         y1[b] = mul_rounded(ct[2 * w + b], E::load(xa)) - mul_rounded(sn, E::load(xb));
         y2[b] = mul_rounded(ct[2 * w + b], E::load(xb)) + mul_rounded(sn, E::load(xa));
       }
-      lo[w] = Mma<E>::pack(y1[0] * qs, y1[1] * qs);  // the one rounding (to nearest even, as E::store rounds)
-      hi[w] = Mma<E>::pack(y2[0] * qs, y2[1] * qs);
+      lo[w] = Mma<E>::pack(y1[0], y1[1]);  // the one rounding (to nearest even, as E::store rounds)
+      hi[w] = Mma<E>::pack(y2[0], y2[1]);
     }
     o0 = make_uint4(lo[0], lo[1], lo[2], lo[3]);
     o1 = make_uint4(hi[0], hi[1], hi[2], hi[3]);
   }
 };
-
-// Eight stored values times a factor, rounded back to storage (pieces of a query that pass through
-// unrotated, or whose rotation rounds on its own terms).
-template <typename E>
-__device__ __forceinline__ uint4 scaled_piece(const uint4& p, float qs) {
-  using S = typename E::storage;
-  uint32_t w[4] = {p.x, p.y, p.z, p.w};
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const float lo = E::load(__builtin_bit_cast(S, (uint16_t)w[k]));
-    const float hi = E::load(__builtin_bit_cast(S, (uint16_t)(w[k] >> 16)));
-    w[k] = Mma<E>::pack(lo * qs, hi * qs);
-  }
-  return make_uint4(w[0], w[1], w[2], w[3]);
-}
 
 // Wait until the matrix pipe has written the results of the products issued from assembly
 // (run32_acc) into the accumulators `o`, before anything but another product touches them.  A

@@ -19,8 +19,9 @@
 //                                        reads (ds_read_b64_tr_b16), each serving all row blocks
 //
 // The loop is a hand-ordered software pipeline: the scores of tile i + 1 run on the matrix pipe
-// under the exponentials of tile i, the products of tile i under the maxima and the score
-// transform of tile i + 1.  Interior tiles of a link take a branch-free ring step.
+// under the exponentials of tile i (each taken of scale * score - reference, formed in fp32 right
+// in front of it), the products of tile i under the maxima of tile i + 1.  Interior tiles of a link
+// take a branch-free ring step, in a loop of their own.
 // V tiles and the staged query tile keep whole rows in LDS, unpadded and swizzled (piece c of row r
 // at position c ^ swz(r)); K tiles land in fragment order (8-token x 128-byte blocks, see the load
 // pattern in the kernel), so that the K reads of a tile share one address register.  The query tile
@@ -199,21 +200,14 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
   const int part_base = item[VA_I_PART_BASE];
   const bool wave_active = (kWaveRows * wave) / G < n_q;  // the wave owns real rows
 
-  float m_ref[kB], m_rel[kB], l_run[kB];  // reference maximum (log2 units), last tile maximum above `base`, row sum
-  // The score products start from -base instead of from zero (and the staged query carries the softmax
-  // scale), so a product's result IS the exponent s * scale - m_ref: base is the row's reference, or 0
-  // while the row has none yet (a reference of -1e30 would swallow the scores).
-  float base[kB], raise_above[kB];  // raise_above = m_ref + kWideRaise - base: what a tile's maximum is tested against
-  va_f32x16 score_start[kB];
+  float m_ref[kB], m_tile[kB], l_run[kB];  // reference maximum (log2 units), last tile maximum, row sum
+  float raise_above[kB];                    // m_ref + kWideRaise: what a tile's maximum is tested against
   va_f32x16 o[kB][kDimTiles];
 #pragma unroll
   for (int b = 0; b < kB; ++b) {
     m_ref[b] = kNegBig;
-    m_rel[b] = kNegBig;
-    base[b] = 0.f;
+    m_tile[b] = kNegBig;
     raise_above[b] = kNegBig + kWideRaise;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) score_start[b][r] = 0.f;
     l_run[b] = 0.f;
 #pragma unroll
     for (int t = 0; t < kDimTiles; ++t)
@@ -342,12 +336,12 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
 #pragma unroll
             for (int jj = 0; jj < kBatch; ++jj) unit[jj].load(a.rope, qh[jj], x, pos[jj]);
 #pragma unroll
-            for (int jj = 0; jj < kBatch; ++jj) unit[jj].finish(a.rope, pos[jj], p0[jj], p1[jj], a.scale_log2);
+            for (int jj = 0; jj < kBatch; ++jj) unit[jj].finish(a.rope, pos[jj], p0[jj], p1[jj]);
           } else {
 #pragma unroll
             for (int jj = 0; jj < kBatch; ++jj) {
-              p0[jj] = scaled_piece<E>(*(const uint4*)(qh[jj] + 8 * c0), a.scale_log2);
-              p1[jj] = scaled_piece<E>(*(const uint4*)(qh[jj] + 8 * c1), a.scale_log2);
+              p0[jj] = *(const uint4*)(qh[jj] + 8 * c0);
+              p1[jj] = *(const uint4*)(qh[jj] + 8 * c1);
             }
           }
 #pragma unroll
@@ -372,8 +366,6 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
             const S* qh = (const S*)a.q + src_row * a.q_row_stride + (long long)(hk * G + g) * kD;
             const Pos3 p = load_pos(a.sub_loc, a.sub_loc_axis_stride, subrow);
             rotated_query_unit<E>(a.rope, qh, x, p, c0, c1, p0, p1);
-            p0 = scaled_piece<E>(p0, a.scale_log2);
-            p1 = scaled_piece<E>(p1, a.scale_log2);
           }
           q_stage[Rl * kChunks + (c0 ^ wide_swz<kD>(Rl))] = va_u32x4{p0.x, p0.y, p0.z, p0.w};
           q_stage[Rl * kChunks + (c1 ^ wide_swz<kD>(Rl))] = va_u32x4{p1.x, p1.y, p1.z, p1.w};
@@ -490,7 +482,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       for (int b = 0; b < kB; ++b) {
         // through the builtin: the compiler sees these products and keeps the wait states between
         // them and the vector-ALU instructions that feed them or read their results
-        into[b] = Mma<E>::run32(kf[s % kKRing], qf[b][s], s == 0 ? score_start[b] : into[b]);
+        into[b] = Mma<E>::run32(kf[s % kKRing], qf[b][s], s == 0 ? va_f32x16{} : into[b]);
       }
       if (s + kKRing < kSteps) read_k_fragment(tile, s + kKRing);
     };
@@ -536,7 +528,11 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       auto exp_piece = [&](int r) __attribute__((always_inline)) {
 #pragma unroll
         for (int b = 0; b < kB; ++b) {
-          cur[b][r] = __builtin_amdgcn_exp2f(cur[b][r]);  // the scores came out of their products as s * scale - m_ref
+          // raw score -> exponent in fp32, as the reference scales its scores.  (The multiply-add sits here,
+          // in the shadow of a score product, rather than under the P.V products, whose slots are full: there
+          // it costs 3.4 % of the kernel, here 0.8 %.  Staging the query times the scale instead makes it
+          // free, but rounds other numbers than the reference does: out of tolerance once scores reach +-20.)
+          cur[b][r] = __builtin_amdgcn_exp2f(fmaf(cur[b][r], a.scale_log2, -m_ref[b]));
           if (r > 0) sum[b] += cur[b][r - 1];
           if (r >= 2 && r % 2 == 0) pw[b][r / 2 - 1] = Mma<E>::pack(cur[b][r - 2], cur[b][r - 1]);
         }
@@ -600,17 +596,16 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
         __builtin_amdgcn_sched_barrier(0);
       }
     };
-    // The reference of the rows is raised to the maxima of the tile in `cur` (m_rel, above base): what was
-    // accumulated against the old reference is rescaled, and so are the tile's scores; the products that
-    // follow start from the new one.
+    // The reference of the rows is raised to the maxima of the tile in `cur` (m_tile, log2 units): what was
+    // accumulated against the old reference is rescaled; the tile's raw scores stay as they are.
     auto raise_reference = [&](int i, auto& cur) __attribute__((always_inline)) {
       accumulator_fence<kB * kDimTiles>(&o[0][0]);
 #pragma unroll
       for (int b = 0; b < kB; ++b) {
-        const float m_new = fmaxf(m_ref[b], m_rel[b] + base[b]);
+        const float m_new = fmaxf(m_ref[b], m_tile[b]);
         const float alpha = __builtin_amdgcn_exp2f(m_ref[b] - m_new);
-        const float step = m_new - base[b];
         m_ref[b] = m_new;
+        raise_above[b] = m_new + kWideRaise;
         l_run[b] *= alpha;
 #pragma unroll
         for (int t = 0; t < kDimTiles; ++t) o[b][t] *= alpha;
@@ -618,12 +613,8 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const bool visible = (t0 + (r / 4) * 8 + 4 * h + (r % 4)) < t_row[b];
-          cur[b][r] = visible ? cur[b][r] - step : -INFINITY;
+          cur[b][r] = visible ? cur[b][r] : -INFINITY;
         }
-        base[b] = m_new > 0.5f * kNegBig ? m_new : 0.f;  // (a row that has seen nothing yet keeps base 0)
-        raise_above[b] = m_new + kWideRaise - base[b];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) score_start[b][r] = -base[b];
       }
     };
     // the test of the steady part: the maxima were gathered under the previous products, nothing is masked
@@ -631,8 +622,8 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
       bool raise = false;
 #pragma unroll
       for (int b = 0; b < kB; ++b) {
-        m_rel[b] = half_wave_max(early_max[b]);
-        raise = raise || m_rel[b] > raise_above[b];
+        m_tile[b] = half_wave_max(early_max[b]) * a.scale_log2;
+        raise = raise || m_tile[b] > raise_above[b];
       }
       return (bool)__any(raise);
     };
@@ -665,16 +656,16 @@ __global__ __launch_bounds__(kWideThreads, 1) void attn_mfma_wide_kernel(AttnArg
             for (int r = 0; r < 16; ++r)
               sc[b][r] = (t0 + (r / 4) * 8 + 4 * h + (r % 4)) < t_row[b] ? sc[b][r] : -INFINITY;
           }
-          // the tile maximum above base: from the maxima found under the previous products, or, for a
-          // masked or first tile, from sc
+          // the tile maximum (raw): from the maxima found under the previous products, or, for a masked or
+          // first tile, from sc
           float tile_max = early_max[b];
           if (masked || !early_max_valid) {
             tile_max = sc[b][0];
 #pragma unroll
             for (int r = 1; r < 16; ++r) tile_max = fmaxf(tile_max, sc[b][r]);
           }
-          m_rel[b] = half_wave_max(tile_max);
-          raise = raise || m_rel[b] > raise_above[b];
+          m_tile[b] = half_wave_max(tile_max) * a.scale_log2;
+          raise = raise || m_tile[b] > raise_above[b];
         }
         raise = __any(raise);
       }

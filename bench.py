@@ -51,11 +51,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # carried here together with the digest of the kernel sources they were measured on
 # (csrc_digest()), and are reported only while that digest is the one of the sources in the tree.
 MEASURED_TRAFFIC = {
-    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_130_005 + 8_988) + 1024 * (17_883 + 512), "csrc": "778986fa809c6eea"},
-    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_098_018 + 4_722) + 1024 * (9_297 + 64), "csrc": "778986fa809c6eea"},
-    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_510_557 + 1024 * 131_393, "csrc": "778986fa809c6eea"},
-    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (439_625 + 1_623_110 + 27_059) + 1024 * (47_445 + 12_397 + 10_624),
-                              "csrc": "778986fa809c6eea"},
+    ("batched_decode", "mfma"): {"bytes": 2 * 1024 * (1_129_938 + 8_988) + 1024 * (17_885 + 512), "csrc": "08c375c61b54cd3d"},
+    ("mrope_decode", "mfma"): {"bytes": 2 * 1024 * (2_098_018 + 4_722) + 1024 * (9_297 + 64), "csrc": "08c375c61b54cd3d"},
+    ("view_prefill", "mfma"): {"bytes": 2 * 1024 * 2_496_982 + 1024 * 131_323, "csrc": "08c375c61b54cd3d"},
+    ("mixed_batch", "mfma"): {"bytes": 2 * 1024 * (439_645 + 1_623_108 + 27_058) + 1024 * (47_429 + 12_397 + 10_624),
+                              "csrc": "08c375c61b54cd3d"},
 }
 
 

@@ -266,11 +266,7 @@ def test_wide_tiles_with_a_late_score_spike(D, dtype, spike):
         a_stored = float(torch.tensor(a, dtype=dtype))  # the planted value as the pool holds it
         want = (seen - spikes + spikes * torch.tensor(a_stored * (D / 2) / D ** 0.5, dtype=torch.float64).exp()).log()
         got = lse.double().cpu()
-        # The wide kernel stages the query times scale * log2(e), rounded once to the storage type (its score
-        # products then come out as exponents): a query of all ones makes that rounding the same in every
-        # dim, so the spike's exponent is off by up to 2^-8 of itself in bf16 (2^-11 in fp16).
-        staged = spike * 0.6931 * 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
-        assert torch.allclose(got, want[:, None].expand_as(got), atol=2e-2 + staged, rtol=0)
+        assert torch.allclose(got, want[:, None].expand_as(got), atol=2e-2, rtol=0)
 
 
 @pytest.mark.parametrize("spike", [15.0, 60.0])
@@ -311,5 +307,4 @@ def test_wide_tiles_with_a_spike_in_the_first_tile_of_a_later_block(D, dtype, sp
     a_stored = float(torch.tensor(a, dtype=dtype))
     want = (seen - 1 + torch.tensor(a_stored * (D / 2) / D ** 0.5, dtype=torch.float64).exp()).log()
     got = lse.double().cpu()
-    staged = spike * 0.6931 * 2.0 ** (-8 if dtype == torch.bfloat16 else -11)  # (the staged query's rounding, see above)
-    assert torch.allclose(got, want[:, None].expand_as(got), atol=2e-2 + staged, rtol=0)
+    assert torch.allclose(got, want[:, None].expand_as(got), atol=2e-2, rtol=0)

@@ -66,6 +66,44 @@ def test_random_prefill_batches(seed):
         run_prefill_parity(op, cpu_pool, dev_pool, specs, 1e4, gen, scale=0.5)
 
 
+def test_random_prefill_batches_with_large_scores():
+    """Keys and queries of standard deviation 2 per element: scores of standard deviation 4 (natural units) that
+    reach +-20 over contexts of a few thousand tokens, so the softmax is close to one-hot and a query rounded
+    anywhere else than where the reference rounds it (say, after a multiplication by the softmax scale) moves
+    the output by far more than the tolerance.  Longer context blocks than the sweeps above: the interior of
+    the wide kernel's walk (its steady loop) does most of the work here."""
+    rng = random.Random(31)
+    for case in range(24):
+        page = rng.choice([1, 4, 16, 16, 16, 32, 64])
+        heads = rng.choice([(4, 4, 64), (8, 2, 64), (8, 2, 128), (16, 2, 128), (8, 2, 256), (16, 4, 256), (16, 1, 256),
+                            (32, 8, 128)])
+        dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+        D = heads[2]
+        rotary = rng.choice([D, D // 2])
+        lens = [rng.choice([5, 33, 257, 400, 777, 1200, 2049, 3100]) for _ in range(rng.randint(1, 4))]
+        reqs = [(rng.choice([1, 33, 64, 100, 150, 260, 500]), rng.choice([0, 3, 16, 200, 333, 1000]))
+                for _ in range(rng.randint(1, 3))]
+        print(f"large-score prefill case {case}: page {page} heads {heads} {dtype} rotary {rotary} blocks {lens} "
+              f"requests {reqs}", flush=True)
+        total_pages = sum(-(-n // page) for n in lens) + sum(-(-(p + n) // page) for n, p in reqs) + 4
+        op, cpu_pool, dev_pool, gen = make_op_and_pool(DEV, dtype, heads, page, total_pages, 1e4, rotary_dim=rotary,
+                                                       seed=31000 + case, scale=2.0, max_pos=8192)
+        blocks, first = [], 0
+        for length in lens:
+            b = CacheBlock(DEV, page)
+            n_pages = -(-length // page)
+            b.grow_pages(torch.arange(first, first + n_pages) * page, length)
+            blocks.append(b)
+            first += n_pages
+        specs = []
+        for n, prefix in reqs:
+            n_pages = -(-(prefix + n) // page)
+            pages = torch.arange(first, first + n_pages, dtype=torch.int32) * page
+            first += n_pages
+            specs.append(PrefillSpec(blocks[rng.randint(0, len(blocks) - 1):], pages, n, prefix))
+        run_prefill_parity(op, cpu_pool, dev_pool, specs, 1e4, gen, scale=2.0)
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_random_decode_views(seed):
     rng = random.Random(seed)
